@@ -8,6 +8,7 @@ from .registry import (
     unregister_architecture,
 )
 from . import llama as _llama  # registers LlamaForCausalLM
+from . import buderax as _buderax  # registers Buderax
 
 __all__ = [
     "Architecture",

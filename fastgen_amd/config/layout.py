@@ -30,14 +30,16 @@ class PartSpec:
 class LayerSpec:
     """One layer: a token mixer and a feed-forward, each with its norm, and
     the name of the arrangement that wires them to the residual stream.
+    ``ffn`` and ``ffn_norm`` may be None: a layer without a feed-forward, or
+    one whose sublayers share the mixer's norm (the arrangement must know).
     ``extra_norms``: further norms by name, for arrangements that own more
     than two (norms after the mixer and the feed-forward, say); the
     arrangement gets them as a dict."""
 
     mixer: PartSpec
-    ffn: PartSpec
+    ffn: Optional[PartSpec]
     mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    ffn_norm: Optional[PartSpec]
     arrangement: str = "pre_norm"
     extra_norms: Mapping[str, PartSpec] = field(default_factory=dict)
 
@@ -50,10 +52,15 @@ class RunEntry:
     by several entries.  Every entry owns storage of its own (pages or a
     state slot) unless ``reads_cache_of`` names an earlier entry of the
     order: then its mixer writes nothing and reads that entry's storage.
+
+    ``inject`` = (index into ``ModelLayout.injections``, pass number): that
+    part adds to the residual stream right before this entry's layer runs
+    (the start of a pass of a looped stretch of layers, say).
     """
 
     layer: int
     reads_cache_of: Optional[int] = None
+    inject: Optional[Tuple[int, int]] = None
 
 
 @dataclass(frozen=True)
@@ -65,9 +72,12 @@ class ModelLayout:
     order: Tuple[RunEntry, ...]
     final_norm: PartSpec
     head: PartSpec
+    injections: Tuple[PartSpec, ...] = ()
 
     def __post_init__(self) -> None:
         for i, e in enumerate(self.order):
+            if e.inject is not None and not 0 <= e.inject[0] < len(self.injections):
+                raise ValueError(f"order[{i}] names injection {e.inject[0]}, which does not exist")
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"order[{i}] names layer {e.layer}, which does not exist")
             if e.reads_cache_of is not None:

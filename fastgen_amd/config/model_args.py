@@ -191,7 +191,9 @@ def read_config_json(model_dir: str | Path) -> dict:
 
 
 def architecture_name(config: Mapping[str, Any]) -> Optional[str]:
-    archs = config.get("architectures")
+    """The name a ``config.json`` gives its model class: the one element of
+    ``architectures``, or the string under ``architecture``."""
+    archs = config.get("architectures", config.get("architecture"))
     if isinstance(archs, (list, tuple)) and len(archs) == 1:
         return archs[0]
     if isinstance(archs, str):

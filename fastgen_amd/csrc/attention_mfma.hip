@@ -1,5 +1,7 @@
 // Paged causal attention on the matrix cores (bf16 in, fp32 accumulate) for
-// gfx950.  Compiled once per head size: -DFG_HD=<multiple of 16, at most 256>.
+// gfx950.  Compiled once per head size: -DFG_HD=<multiple of 16, at most 256>;
+// with -DFG_EXACT_P the softmax weights keep 16 significant bits in the product
+// with the values (for models that ask for weights of more than bfloat16).
 //
 // Both kernels work on *items*: an item is a run of consecutive query tokens
 // of one sequence; its rows are (token, query head of one kv head's group),
@@ -154,6 +156,11 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], co
     for (int db = 0; db < NDB; ++db) vop1[db] = load_v(db, 1);
   }
   bf16x8 pop[RB][2];
+#ifdef FG_EXACT_P
+  // The weights enter the product with the values as the sum of two bfloat16 terms (what the first
+  // rounding drops is the second): 16 significant bits instead of 8, for twice the MFMAs of that product.
+  bf16x8 pop_lo[RB][2];
+#endif
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     float mx = -INFINITY;
@@ -182,6 +189,9 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], co
         const float p = __builtin_amdgcn_exp2f(fmaf(s[rb][kb][i], scale_log2, -m_use));
         sum += p;
         pop[rb][kb >> 1][4 * (kb & 1) + i] = (__bf16)p;
+#ifdef FG_EXACT_P
+        pop_lo[rb][kb >> 1][4 * (kb & 1) + i] = (__bf16)(p - (float)(__bf16)p);
+#endif
       }
     l[rb] = l[rb] * alpha + sum;  // this lane's share of the row's sum; the groups are added at the end
     // once the maxima have settled no row of the wave changes its maximum: nothing to rescale then
@@ -197,8 +207,12 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], co
     for (int db = 0; db < NDB; ++db) {
       const bf16x8 v = PREFETCH ? (ks == 0 ? vop0[db] : vop1[db]) : load_v(db, ks);
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
+      for (int rb = 0; rb < RB; ++rb) {
         o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pop[rb][ks], o[rb][db], 0, 0, 0);
+#ifdef FG_EXACT_P
+        o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pop_lo[rb][ks], o[rb][db], 0, 0, 0);
+#endif
+      }
     }
 }
 

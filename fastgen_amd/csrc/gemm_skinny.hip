@@ -147,6 +147,8 @@ struct RopeKv {
   bf16_t* k_pages;
   bf16_t* v_pages;
   int n_heads, n_kv, hd, rotary_dim, page_size;
+  int v_from_k;   // w has no v rows: a token's value is its key before the rotation
+  int gate_cols;  // w ends with this many rows of an output gate: y[m][n_heads * hd + j] = sigmoid(gate j)
 };
 
 __device__ __forceinline__ bf16x8 gs_zero8() {
@@ -314,7 +316,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
       a *= rscale[m];
       b *= rscale[m];
       const int q_cols = rk.n_heads * rk.hd, k_cols = rk.n_kv * rk.hd;
+      const int gate_start = q_cols + (rk.v_from_k ? k_cols : 2 * k_cols);
       const int d = n % rk.hd;
+      const float a0 = a, b0 = b;  // as projected
       if (n < q_cols + k_cols && rk.table && d < rk.rotary_dim) {
         const float cs = rk.table[((size_t)m * (rk.rotary_dim / 2) + d / 2) * 2];
         const float sn = rk.table[((size_t)m * (rk.rotary_dim / 2) + d / 2) * 2 + 1];
@@ -328,6 +332,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
         *(bf16x2_t*)((bf16_t*)y + (size_t)m * ldy + n) = v2;
         continue;
       }
+      if (n >= gate_start) {
+        bf16x2_t v2 = {(__bf16)__frcp_rn(1.f + __expf(-a)), (__bf16)__frcp_rn(1.f + __expf(-b))};
+        *(bf16x2_t*)((bf16_t*)y + (size_t)m * ldy + q_cols + (n - gate_start)) = v2;
+        continue;
+      }
       const int slot = rk.slots[m];
       if (slot < 0) continue;
       const KvLayout lay(rk.page_size, rk.hd);
@@ -337,6 +346,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
         const int kvh = (n - q_cols) / rk.hd;
         bf16x2_t v2 = {(__bf16)a, (__bf16)b};
         *(bf16x2_t*)(rk.k_pages + ((size_t)page * rk.n_kv + kvh) * head_elems + lay.k_off(off, d)) = v2;
+        if (rk.v_from_k) {
+          bf16_t* vh = rk.v_pages + ((size_t)page * rk.n_kv + kvh) * head_elems;
+          vh[lay.v_off(off, d)] = (bf16_t)a0;
+          vh[lay.v_off(off, d + 1)] = (bf16_t)b0;
+        }
       } else {
         const int kvh = (n - q_cols - k_cols) / rk.hd;
         bf16_t* vh = rk.v_pages + ((size_t)page * rk.n_kv + kvh) * head_elems;
@@ -594,22 +608,26 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
 // q, k, v projections of at most 16 rows with the rotation and the cache write in the epilogue:
 // w = [q rows; k rows; v rows] ([(H + 2 KV) * hd, K]); y = rotated q [M, H * hd]; rotated k and v go
 // to slots[m] of the pages.  table: cos/sin of the rows' positions (null: no rotation).
+// v_from_k: w has no v rows and the k columns, before their rotation, are the values.  gate_cols (0 or
+// H * hd): w ends with the rows of an output gate, whose sigmoid goes to y[m][H * hd ..].
 // ssq [M, n_parts] (null: x is taken as it is): the rows' sums of squares for the norm folded into this product.
 extern "C" int fg_gemm_skinny_qkv(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int K,
                                   const float* table, const int* slots, void* k_pages, void* v_pages,
-                                  int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
-                                  const float* ssq, int n_parts, int dim, float eps, hipStream_t stream) {
+                                  int n_heads, int n_kv, int hd, int rotary_dim, int page_size, int v_from_k,
+                                  int gate_cols, const float* ssq, int n_parts, int dim, float eps,
+                                  hipStream_t stream) {
   if (M <= 0) return FG_OK;
-  const int N = (n_heads + 2 * n_kv) * hd;
+  if (gate_cols < 0 || gate_cols % 16) return FG_ERR_ARG;
+  const int N = (n_heads + (v_from_k ? 1 : 2) * n_kv) * hd + gate_cols;
   if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K) || hd % 16 || n_heads <= 0 ||
       n_kv <= 0 || rotary_dim < 0 || rotary_dim > hd || rotary_dim % 2 || page_size <= 0 || page_size % 8 ||
-      ldy < n_heads * hd || ldy % 2 || !slots || !k_pages || !v_pages || (rotary_dim && !table) ||
+      ldy < n_heads * hd + gate_cols || ldy % 2 || !slots || !k_pages || !v_pages || (rotary_dim && !table) ||
       (ssq && (n_parts < 1 || dim < 1 || !(eps >= 0.f))))
     return FG_ERR_ARG;
   const RowScale sc{ssq, n_parts, ssq ? 1.f / (float)dim : 0.f, eps};
   const Residual rs{};
   const RopeKv rk{rotary_dim ? table : nullptr, slots, (bf16_t*)k_pages, (bf16_t*)v_pages,
-                  n_heads, n_kv, hd, rotary_dim, page_size};
+                  n_heads, n_kv, hd, rotary_dim, page_size, v_from_k, gate_cols};
   const int blocks = N / 16;
   if (blocks >= 1024)
     gemm_skinny16_kernel<4, EPI_ROPE_KV, bf16_t><<<blocks, 256, 0, stream>>>(

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
     const float* __restrict__ freqs, const float* __restrict__ table, const int* __restrict__ slots,
     T* __restrict__ k_pages,
     T* __restrict__ v_pages, int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
-    int write_kv) {
+    int write_kv, int v_col) {
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * row_stride;
   const float pos = (float)positions[t];
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
     }
   }
   if (slot >= 0) {
-    const T* v = row + (size_t)(n_heads + n_kv) * hd;
+    const T* v = row + v_col;
     for (int e = threadIdx.x; e < n_kv * hd; e += ROPE_THREADS) {
       const int kvh = e / hd, d = e % hd;
       v_pages[((size_t)page * n_kv + kvh) * head_elems + lay.v_off(off, d)] = v[e];
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
     const float* __restrict__ freqs, const float* __restrict__ table, const int* __restrict__ slots,
     T* __restrict__ k_pages,
     T* __restrict__ v_pages, int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
-    int write_kv) {
+    int write_kv, int v_col) {
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * row_stride;
   const float pos = (float)positions[t];
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
   if (slot >= 0) {
     // v: one element a thread, consecutive threads consecutive head dims: in the transposed page
     // these lie 16 bytes apart, so a wave's store stays within a few cache lines
-    const T* v = row + (size_t)(n_heads + n_kv) * hd;
+    const T* v = row + v_col;
     for (int e = threadIdx.x; e < n_kv * hd; e += ROPE_THREADS) {
       const int kvh = e / hd, d = e % hd;
       v_pages[((size_t)page * n_kv + kvh) * head_elems + lay.v_off(off, d)] = v[e];
@@ -164,23 +164,27 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
 // row.  With write_kv == 0 only q is rotated (a mixer that reads another
 // layer's cache).
 // `table` (from fg_rope_table, for the same positions) replaces the sin/cos
-// of `freqs` when given.
+// of `freqs` when given.  v_col: the column of a row at which the values begin:
+// (n_heads + n_kv) * hd where they have a projection of their own, n_heads * hd
+// where a token's value is its key before the rotation (the k columns of the row
+// are never written: the rotated keys go to the pages only).
 extern "C" int fg_rope_kv_write(void* qkv, int row_stride, const int* positions,
                                 const float* freqs, const float* table, const int* slots, void* k_pages,
                                 void* v_pages, int n_tokens, int n_heads, int n_kv, int hd,
-                                int rotary_dim, int page_size, int write_kv, int dtype,
+                                int rotary_dim, int page_size, int write_kv, int v_col, int dtype,
                                 hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
   if (hd <= 0 || hd % 2 || rotary_dim < 0 || rotary_dim > hd || rotary_dim % 2 ||
       page_size <= 0 || n_heads <= 0 || n_kv < 0)
     return FG_ERR_ARG;
   if (write_kv && (hd % 8 || page_size % 8)) return FG_ERR_ARG;  // the page layout is in chunks of 8
-  if (row_stride < (n_heads + (write_kv ? 2 * n_kv : 0)) * hd) return FG_ERR_ARG;
+  if (row_stride < (n_heads + (write_kv ? n_kv : 0)) * hd) return FG_ERR_ARG;
+  if (write_kv && (v_col < n_heads * hd || v_col % 8 || row_stride < v_col + n_kv * hd)) return FG_ERR_ARG;
   const bool vec = hd % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 8 == 0;
 #define LAUNCH(T, KERNEL)                                                                         \
   KERNEL<T><<<n_tokens, ROPE_THREADS, 0, stream>>>((T*)qkv, row_stride, positions, freqs, table,  \
                                                    slots, (T*)k_pages, (T*)v_pages, n_heads, n_kv, \
-                                                   hd, rotary_dim, page_size, write_kv)
+                                                   hd, rotary_dim, page_size, write_kv, v_col)
   if (dtype == FG_F32) {
     if (vec) LAUNCH(float, rope_kv_write_vec_kernel); else LAUNCH(float, rope_kv_write_kernel);
   } else if (dtype == FG_BF16) {

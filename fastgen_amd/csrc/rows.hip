@@ -13,26 +13,114 @@
 template <class TW>
 __global__ __launch_bounds__(ROWS_THREADS) void embed_kernel(
     const TW* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ out,
-    int dim, int vocab) {
+    int dim, int vocab, float scale) {
   const int t = blockIdx.x;
   int tok = tokens[t];
   // ids are validated on the host; the clamp only keeps a bad id from faulting
   tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
   const TW* src = table + (size_t)tok * dim;
   float* dst = out + (size_t)t * dim;
-  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) dst[i] = to_f<TW>(src[i]);
+  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) dst[i] = to_f<TW>(src[i]) * scale;
 }
 
 extern "C" int fg_embed(const void* table, int table_dtype, const int* tokens, float* out,
-                        int n_tokens, int dim, int vocab, hipStream_t stream) {
+                        int n_tokens, int dim, int vocab, float scale, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
   if (dim <= 0 || vocab <= 0) return FG_ERR_ARG;
   if (table_dtype == FG_F32)
-    embed_kernel<float><<<n_tokens, ROWS_THREADS, 0, stream>>>((const float*)table, tokens, out, dim, vocab);
+    embed_kernel<float><<<n_tokens, ROWS_THREADS, 0, stream>>>((const float*)table, tokens, out, dim, vocab, scale);
   else if (table_dtype == FG_BF16)
-    embed_kernel<bf16_t><<<n_tokens, ROWS_THREADS, 0, stream>>>((const bf16_t*)table, tokens, out, dim, vocab);
+    embed_kernel<bf16_t><<<n_tokens, ROWS_THREADS, 0, stream>>>((const bf16_t*)table, tokens, out, dim, vocab, scale);
   else
     return FG_ERR_ARG;
+  return fg_launch_status();
+}
+
+// -------------------------------------------------- additions to the stream
+// h[t] = ((h[t] + delta[t]) + again[t]) + row, all fp32, in that order: what a layer left to be added
+// (rows of the activation dtype, or fp32 partial sums in order), then rows that enter the stream once
+// more (the embedding's output), then one vector for all tokens.  Each of the three may be absent.
+template <class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void stream_add_kernel(
+    float* __restrict__ h, const TA* __restrict__ delta, const float* __restrict__ parts, int n_parts,
+    size_t part_stride, const float* __restrict__ again, const float* __restrict__ row, int dim) {
+  const size_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) {
+    float v = h[t * dim + i];
+    if (delta) v += to_f<TA>(delta[t * dim + i]);
+    if (parts)
+      for (int p = 0; p < n_parts; ++p) v += parts[p * part_stride + t * dim + i];
+    if (again) v += again[t * dim + i];
+    if (row) v += row[i];
+    h[t * dim + i] = v;
+  }
+}
+
+extern "C" int fg_stream_add(float* h, const void* delta, int delta_dtype, const float* parts, int n_parts,
+                             long long part_stride, const float* again, const float* row, int n_rows, int dim,
+                             hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (dim <= 0 || (parts && n_parts < 1)) return FG_ERR_ARG;
+  if (delta_dtype == FG_F32)
+    stream_add_kernel<float><<<n_rows, ROWS_THREADS, 0, stream>>>(h, (const float*)delta, parts, n_parts,
+                                                                  (size_t)part_stride, again, row, dim);
+  else if (delta_dtype == FG_BF16)
+    stream_add_kernel<bf16_t><<<n_rows, ROWS_THREADS, 0, stream>>>(h, (const bf16_t*)delta, parts, n_parts,
+                                                                   (size_t)part_stride, again, row, dim);
+  else
+    return FG_ERR_ARG;
+  return fg_launch_status();
+}
+
+// out[t] = a[t] + b[t] in fp32 (two sublayers' outputs that go to the stream as one sum)
+template <class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void add_rows_kernel(const TA* __restrict__ a, const TA* __restrict__ b,
+                                                                float* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * ROWS_THREADS + threadIdx.x;
+  if (i < n) out[i] = to_f<TA>(a[i]) + to_f<TA>(b[i]);
+}
+
+extern "C" int fg_add_rows(const void* a, const void* b, float* out, long long n, int dtype, hipStream_t stream) {
+  if (n <= 0) return FG_OK;
+  const unsigned blocks = (unsigned)((n + ROWS_THREADS - 1) / ROWS_THREADS);
+  if (dtype == FG_F32)
+    add_rows_kernel<float><<<blocks, ROWS_THREADS, 0, stream>>>((const float*)a, (const float*)b, out, (size_t)n);
+  else if (dtype == FG_BF16)
+    add_rows_kernel<bf16_t><<<blocks, ROWS_THREADS, 0, stream>>>((const bf16_t*)a, (const bf16_t*)b, out, (size_t)n);
+  else
+    return FG_ERR_ARG;
+  return fg_launch_status();
+}
+
+// x[t][i] *= sigmoid(g[t][i]) (or g[t][i] itself when the sigmoid was taken where g was made), fp32
+// inside, one rounding.  Rows of x and g have strides of their own (g may be columns of a wider product).
+template <class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void gate_mul_kernel(TA* __restrict__ x, int ldx, const TA* __restrict__ g,
+                                                                int ldg, int width, int sigmoid) {
+  const size_t t = blockIdx.y;
+  const int i = blockIdx.x * ROWS_THREADS + threadIdx.x;
+  if (i >= width) return;
+  float gv = to_f<TA>(g[t * ldg + i]);
+  if (sigmoid) gv = 1.f / (1.f + expf(-gv));
+  x[t * ldx + i] = from_f<TA>(to_f<TA>(x[t * ldx + i]) * gv);
+}
+
+extern "C" int fg_gate_mul(void* x, int ldx, const void* g, int ldg, int n_rows, int width, int sigmoid, int dtype,
+                           hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (width <= 0 || ldx < width || ldg < width) return FG_ERR_ARG;
+  for (int r0 = 0; r0 < n_rows; r0 += 65535) {
+    const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    dim3 grid((width + ROWS_THREADS - 1) / ROWS_THREADS, nr);
+    if (dtype == FG_F32)
+      gate_mul_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>((float*)x + (size_t)r0 * ldx, ldx,
+                                                                (const float*)g + (size_t)r0 * ldg, ldg, width, sigmoid);
+    else if (dtype == FG_BF16)
+      gate_mul_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((bf16_t*)x + (size_t)r0 * ldx, ldx,
+                                                                 (const bf16_t*)g + (size_t)r0 * ldg, ldg, width, sigmoid);
+    else
+      return FG_ERR_ARG;
+  }
   return fg_launch_status();
 }
 

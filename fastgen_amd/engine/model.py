@@ -9,7 +9,7 @@ The reference's counterpart is the weight-only ``Transformer`` skeleton
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Any, Dict, List, Mapping, Optional, Sequence
 
@@ -33,6 +33,7 @@ class ModelParts:
     final_norm: Any
     head: Any
     all_parts: List[Any]
+    injections: List[Any] = field(default_factory=list)
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self.all_parts for s in p.tensor_specs()]
@@ -47,18 +48,19 @@ def build_parts(layout: ModelLayout) -> ModelParts:
     blocks, mixers, parts = [], [], [embed]
     for ls in layout.layers:
         mixer = build_part("mixer", ls.mixer)
-        ffn = build_part("feed_forward", ls.ffn)
+        ffn = build_part("feed_forward", ls.ffn) if ls.ffn is not None else None
         n1 = build_part("norm", ls.mixer_norm)
-        n2 = build_part("norm", ls.ffn_norm)
+        n2 = build_part("norm", ls.ffn_norm) if ls.ffn_norm is not None else None
         extra = {name: build_part("norm", spec) for name, spec in ls.extra_norms.items()}
         # an arrangement that asks for no further norms is built from the four parts alone
         blocks.append(build_part("arrangement", PartSpec(ls.arrangement), mixer, ffn, n1, n2, *([extra] if extra else [])))
         mixers.append(mixer)
-        parts += [mixer, ffn, n1, n2, *extra.values()]
+        parts += [p for p in (mixer, ffn, n1, n2, *extra.values()) if p is not None]
+    injections = [build_part("injection", spec) for spec in layout.injections]
     final_norm = build_part("norm", layout.final_norm)
     head = build_part("head", layout.head)
-    parts += [final_norm, head]
-    return ModelParts(layout, embed, blocks, mixers, final_norm, head, parts)
+    parts += [*injections, final_norm, head]
+    return ModelParts(layout, embed, blocks, mixers, final_norm, head, parts, injections)
 
 
 class Model:
@@ -163,13 +165,20 @@ class Model:
         if not self.loaded:
             raise RuntimeError("the model has no weights yet")
         h = self.parts.embed.forward(ctx.tokens, ctx)
+        injections = self.parts.injections
+        # the embedding's output as it was, for injections that add it again (h itself moves on)
+        embedded = h.clone() if any(p.needs_embedding for p in injections) else None
         pending = None  # rows still to be added to h, or ScaledRows (added already, the next norm half done)
         blocks, order = self.parts.blocks, self.layout.order
         for i, entry in enumerate(order):
             block = blocks[entry.layer]
+            if entry.inject is not None:
+                injections[entry.inject[0]].forward(h, None if isinstance(pending, ScaledRows) else pending,
+                                                    embedded, entry.inject[1])
+                pending = None
             if getattr(block, "folds_norms", False):
                 # the norm that follows this block is the next block's first, if that block can take over
-                after = blocks[order[i + 1].layer] if i + 1 < len(order) else None
+                after = blocks[order[i + 1].layer] if i + 1 < len(order) and order[i + 1].inject is None else None
                 next_norm = after.mixer_norm if getattr(after, "folds_norms", False) else None
                 pending = block.forward(h, pending, ctx, stores[i], next_norm=next_norm)
             else:

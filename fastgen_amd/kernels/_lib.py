@@ -44,11 +44,14 @@ LIBRARIES: Dict[str, str] = {
     "gemm_skinny": "gemm_skinny.hip",
     "gemm_tiled": "gemm_tiled.hip",
     "sampling": "sampling.hip",
+    "moe": "moe.hip",
 }
 
-# libraries compiled once per value of a macro: name -> (source, macro, values that build_all compiles)
+# libraries compiled once per value of a macro: name -> (source, macro, values that build_all compiles,
+# further defines)
 VARIANT_LIBRARIES: Dict[str, tuple] = {
-    "attention_mfma": ("attention_mfma.hip", "FG_HD", tuple(range(16, 257, 16))),
+    "attention_mfma": ("attention_mfma.hip", "FG_HD", tuple(range(16, 257, 16)), ()),
+    "attention_mfma_exact": ("attention_mfma.hip", "FG_HD", tuple(range(16, 257, 16)), ("-DFG_EXACT_P=1",)),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -77,8 +80,8 @@ def _split_variant(name: str):
     """``attention_mfma@128`` -> (source file, ["-DFG_HD=128"], file stem)."""
     if "@" in name:
         base, value = name.split("@", 1)
-        src, macro, _ = VARIANT_LIBRARIES[base]
-        return src, [f"-D{macro}={int(value)}"], f"{base}_{int(value)}"
+        src, macro, _, more = VARIANT_LIBRARIES[base]
+        return src, [f"-D{macro}={int(value)}", *more], f"{base}_{int(value)}"
     return LIBRARIES[name], [], name
 
 
@@ -171,7 +174,7 @@ def build_all(*, force: bool = True, verbose: bool = True, jobs: int = 8) -> Dic
     """Compile every kernel library (``force``: also those already built)."""
     from concurrent.futures import ThreadPoolExecutor
 
-    every = list(LIBRARIES) + [f"{b}@{v}" for b, (_, _, values) in VARIANT_LIBRARIES.items() for v in values]
+    every = list(LIBRARIES) + [f"{b}@{v}" for b, (_, _, values, _) in VARIANT_LIBRARIES.items() for v in values]
     names = [n for n in every if force or find_built(n) is None]
     out = {n: find_built(n) for n in every if n not in names}
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:

@@ -90,8 +90,8 @@ def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
 
 
 # --------------------------------------------------------------------- rows
-def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t] = table[tokens[t]] as fp32 (``fastgen/forward.py:406-409``)."""
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[tokens[t]] * scale as fp32 (``fastgen/forward.py:406-409``, which has no scale)."""
     _gpu(table, tokens, out)
     n = tokens.numel()
     _need(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [vocab, dim]")
@@ -99,7 +99,8 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch
     _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (n, table.shape[1]),
           "out must be contiguous float32 [n_tokens, dim]")
     st = _lib.load("rows").fg_embed(
-        _ptr(table), _code(table), _ptr(tokens), _ptr(out), n, table.shape[1], table.shape[0], _stream(out))
+        _ptr(table), _code(table), _ptr(tokens), _ptr(out), n, table.shape[1], table.shape[0],
+        ctypes.c_float(scale), _stream(out))
     _check(st, "embed")
     return out
 
@@ -135,6 +136,63 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         _ptr(rows), n_rows, dim, ctypes.c_float(eps), _code(out), _code(weight), _stream(out))
     _check(st, "add_rmsnorm")
     return out
+
+
+def _delta_args(h: torch.Tensor, delta: Optional[torch.Tensor], what: str):
+    """C arguments (delta, dtype code, parts, n_parts, part stride) for what is to be added to the fp32
+    stream ``h``: nothing, rows ``[T, dim]``, or fp32 partial sums ``[S, T, dim]``."""
+    if delta is None:
+        return _ptr(None), F32, _ptr(None), 0, ctypes.c_longlong(0)
+    if delta.dim() == 3:
+        _need(delta.dtype == torch.float32 and delta.shape[1:] == h.shape and delta.stride(2) == 1
+              and delta.stride(1) == h.shape[1], f"{what}: partial sums must be float32 [S, T, dim] with contiguous rows")
+        return _ptr(None), F32, _ptr(delta), delta.shape[0], ctypes.c_longlong(delta.stride(0))
+    _need(delta.shape == h.shape and delta.is_contiguous(), f"{what}: delta must be contiguous and shaped like h")
+    return _ptr(delta), _code(delta), _ptr(None), 0, ctypes.c_longlong(0)
+
+
+def stream_add(h: torch.Tensor, delta: Optional[torch.Tensor], again: Optional[torch.Tensor],
+               row: Optional[torch.Tensor]) -> torch.Tensor:
+    """``h = ((h + delta) + again) + row`` in place on the fp32 stream ``h [T, dim]``, in that order:
+    ``delta`` as :func:`add_rmsnorm` takes it, ``again`` fp32 ``[T, dim]``, ``row`` fp32 ``[dim]`` for
+    every token.  Each may be None."""
+    _gpu(h, delta, again, row)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [T, dim]")
+    T, dim = h.shape
+    if again is not None:
+        _need(again.dtype == torch.float32 and again.shape == h.shape and again.is_contiguous(),
+              "again must be contiguous float32, shaped like h")
+    if row is not None:
+        _need(row.dtype == torch.float32 and row.shape == (dim,) and row.is_contiguous(), "row must be float32 [dim]")
+    st = _lib.load("rows").fg_stream_add(_ptr(h), *_delta_args(h, delta, "stream_add"), _ptr(again), _ptr(row), T, dim,
+                                         _stream(h))
+    _check(st, "stream_add")
+    return h
+
+
+def add_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``a + b`` of two ``[T, dim]`` tensors of one dtype as fp32 ``[1, T, dim]``: two sublayers' outputs
+    as the one sum that a norm adds to the stream."""
+    _gpu(a, b)
+    _need(a.dim() == 2 and a.shape == b.shape and a.dtype == b.dtype and a.is_contiguous() and b.is_contiguous(),
+          "a and b must be contiguous [T, dim] of one dtype")
+    out = torch.empty((1, *a.shape), dtype=torch.float32, device=a.device)
+    st = _lib.load("rows").fg_add_rows(_ptr(a), _ptr(b), _ptr(out), ctypes.c_longlong(a.numel()), _code(a), _stream(a))
+    _check(st, "add_rows")
+    return out
+
+
+def gate_mul(x: torch.Tensor, gate: torch.Tensor, sigmoid: bool = True) -> torch.Tensor:
+    """``x *= sigmoid(gate)`` in place (``x *= gate`` with ``sigmoid=False``); ``x`` and ``gate`` are
+    ``[T, width]`` with unit column stride and row strides of their own."""
+    _gpu(x, gate)
+    _need(x.dim() == 2 and gate.dim() == 2 and x.shape[0] == gate.shape[0] and gate.shape[1] >= x.shape[1]
+          and x.dtype == gate.dtype and x.stride(1) == 1 and gate.stride(1) == 1,
+          "x [T, width] and gate [T, >= width] must share a dtype and have unit column stride")
+    st = _lib.load("rows").fg_gate_mul(_ptr(x), x.stride(0), _ptr(gate), gate.stride(0), x.shape[0], x.shape[1],
+                                       int(sigmoid), _code(x), _stream(x))
+    _check(st, "gate_mul")
+    return x
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -196,16 +254,21 @@ def rope_table(positions: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[torch.Tensor],
                   slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
                   v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
-                  rotary_dim: int, write_kv: bool = True, table: Optional[torch.Tensor] = None) -> None:
+                  rotary_dim: int, write_kv: bool = True, table: Optional[torch.Tensor] = None,
+                  v_col: Optional[int] = None) -> None:
     """Rotate q and k of ``qkv [T, (H+2KV)*hd]`` in place and store k, v at
     ``slots`` of the paged cache (K pages ``[n_pages, KV, P, hd]``, V pages
     ``[n_pages, KV, hd, P]``).  ``kernels/rope.py:56-89``, ``forward.py:449-460``.
+    ``v_col``: the column at which a row's values begin (default: behind the keys);
+    ``n_heads * head_dim`` makes a token's value its key before the rotation.
     """
     _gpu(qkv, positions, freqs, slots, k_pages, v_pages)
     _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be [T, width] with unit column stride")
     T = qkv.shape[0]
-    width = (n_heads + (2 * n_kv if write_kv else 0)) * head_dim
+    v_col = (n_heads + n_kv) * head_dim if v_col is None else int(v_col)
+    width = max((n_heads + n_kv) * head_dim, v_col + n_kv * head_dim) if write_kv else n_heads * head_dim
     _need(qkv.shape[1] >= width, f"qkv rows hold {qkv.shape[1]} elements, {width} are needed")
+    _need(v_col >= n_heads * head_dim and v_col % 8 == 0, "the values begin behind the queries, at a multiple of 8")
     _i32(positions, "positions", T)
     _need(head_dim % 2 == 0 and 0 <= rotary_dim <= head_dim and rotary_dim % 2 == 0,
           "head_dim and rotary_dim must be even and rotary_dim <= head_dim")
@@ -229,7 +292,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[to
     st = _lib.load("rope_kv").fg_rope_kv_write(
         _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(freqs), _ptr(table if rotary_dim else None), _ptr(slots),
         _ptr(k_pages), _ptr(v_pages),
-        T, n_heads, n_kv, head_dim, rotary_dim, page_size, int(write_kv), _code(qkv), _stream(qkv))
+        T, n_heads, n_kv, head_dim, rotary_dim, page_size, int(write_kv), v_col, _code(qkv), _stream(qkv))
     _check(st, "rope_kv_write")
 
 
@@ -366,7 +429,8 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
                          plan: Optional[torch.Tensor] = None, max_chunks: Optional[int] = None,
-                         min_tiles: int = 4, max_rows: int = 16, tile_rows: Optional[int] = None) -> torch.Tensor:
+                         min_tiles: int = 4, max_rows: int = 16, tile_rows: Optional[int] = None,
+                         exact_weights: bool = False) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``small_items`` / ``big_items`` are
     device int32 ``[n, 4]`` lists from :func:`attention_items` (16-byte aligned);
     every query token of the step must be covered by exactly one item.
@@ -376,7 +440,8 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
     rows the big items were cut for (:func:`attention_tile_rows`; default: the larger form's).
     With items of both kinds the tile kernel runs on a second stream beside the split kernel and
     the current stream waits for it before this returns (not while a graph is captured, not with
-    ``FG_ONE_STREAM=1``)."""
+    ``FG_ONE_STREAM=1``).  ``exact_weights``: the build of the kernels in which the softmax weights enter
+    the product with the values as two bfloat16 terms (16 significant bits)."""
     _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items, plan)
     n_pages, n_kv, page_size, hd = k_pages.shape
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
@@ -392,7 +457,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
     _need(out.shape == (T, n_heads * hd) and out.stride(1) == 1 and out.stride(0) % 4 == 0, "out must be [T, H*hd]")
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1,
           "block_table must be int32 [B, max_pages]")
-    lib = _lib.load(f"attention_mfma@{hd}")
+    lib = _lib.load(f"attention_mfma_exact@{hd}" if exact_weights else f"attention_mfma@{hd}")
     G = n_heads // n_kv
     beside = None
     if (small_items is not None and small_items.numel() and big_items is not None and big_items.numel()
@@ -438,8 +503,10 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
 
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
-                    group, ctx, n_heads: int, scale: float, window: int = 0) -> torch.Tensor:
+                    group, ctx, n_heads: int, scale: float, window: int = 0,
+                    exact_weights: bool = False) -> torch.Tensor:
     """Attention for one step: picks the kernel for the step's dtype and shape.
+    ``exact_weights``: see :func:`paged_attention_mfma` (the general kernel's weights are fp32 anyway).
 
     ``group`` carries the block table of the layer's cache group, ``ctx`` the
     step's per-token vectors (``fastgen_amd.engine.context``).  bfloat16 with a
@@ -484,7 +551,8 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
     # rows of the largest small item: one token a sequence in a decode step (also a captured one)
     rows = G * int(ctx.q_lens.max()) if big_d is None else 16
     return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
-                                window, split_plan, chunks, max_rows=min(16, rows), tile_rows=tile_rows)
+                                window, split_plan, chunks, max_rows=min(16, rows), tile_rows=tile_rows,
+                                exact_weights=exact_weights)
 
 
 # ----------------------------------------------------------------------- gemm
@@ -740,11 +808,13 @@ def gemm_tiled(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None,
 
 def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor,
                     k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
-                    rotary_dim: int) -> torch.Tensor:
+                    rotary_dim: int, value_from_key: bool = False, gate: bool = False) -> torch.Tensor:
     """The q, k, v projections of at most 16 rows with :func:`rope_kv_write` in
     the product's epilogue: returns the rotated queries ``[M, H*hd]``; the rotated
     keys and the values go straight into their cache pages.  ``x`` may be :class:`ScaledRows`, ``wqkv`` a
-    matrix or :class:`PackedWeight`."""
+    matrix or :class:`PackedWeight`.  ``value_from_key``: ``wqkv`` has no v rows, a token's value is its
+    key before the rotation.  ``gate``: ``wqkv`` ends with ``H*hd`` rows of an output gate, and the result
+    is ``[M, 2*H*hd]``: the queries, then the sigmoid of the gate."""
     scaled = x if isinstance(x, ScaledRows) else None
     if scaled is not None:
         x = scaled.rows
@@ -754,7 +824,9 @@ def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor,
     _need(x.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16,
           "gemm_skinny_qkv takes bfloat16")
     w_ptr, ldw = _weight_args(wqkv, K, "gemm_skinny_qkv")
-    _need(0 < M <= 16 and tuple(wqkv.shape) == ((n_heads + 2 * n_kv) * head_dim, K), "x [M<=16, K], wqkv [(H+2KV)*hd, K]")
+    gate_cols = n_heads * head_dim if gate else 0
+    n_rows = (n_heads + (1 if value_from_key else 2) * n_kv) * head_dim + gate_cols
+    _need(0 < M <= 16 and tuple(wqkv.shape) == (n_rows, K), f"x [M<=16, K], wqkv [{n_rows}, K]")
     _need(K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0,
           "K must be a multiple of 8, rows 16-byte aligned")
     _need(head_dim % 16 == 0, "head size must be a multiple of 16")
@@ -765,11 +837,11 @@ def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor,
     if rotary_dim:
         _need(table is not None and table.dtype == torch.float32 and table.is_contiguous()
               and table.shape == (M, rotary_dim // 2, 2), "table must be float32 [M, rotary_dim/2, 2]")
-    q = torch.empty((M, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    q = torch.empty((M, n_heads * head_dim + gate_cols), dtype=torch.bfloat16, device=x.device)
     st = _lib.load("gemm_skinny").fg_gemm_skinny_qkv(
         _ptr(x), x.stride(0), w_ptr, ldw, _ptr(q), q.stride(0), M, K,
         _ptr(table if rotary_dim else None), _ptr(slots), _ptr(k_pages), _ptr(v_pages), n_heads, n_kv, head_dim,
-        rotary_dim, page_size, *_row_scale_args(scaled, M), _stream(x))
+        rotary_dim, page_size, int(value_from_key), gate_cols, *_row_scale_args(scaled, M), _stream(x))
     _check(st, "gemm_skinny_qkv")
     return q
 
@@ -815,4 +887,117 @@ def logprob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
     out = torch.empty((n,), dtype=torch.float32, device=logits.device)
     st = _lib.load("sampling").fg_logprob(_ptr(logits), logits.stride(0), n, V, _ptr(tokens), _ptr(out), _stream(logits))
     _check(st, "logprob")
+    return out
+
+
+# ------------------------------------------------------------- routed experts
+MOE_TILE_ROWS = (16, 32, 64)  # rows of one expert that a tile of the matrix-core kernels holds
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """Per row of ``x [T, dim]``: fp32 logits ``x router^T + bias`` (``router`` fp32 ``[E, dim]``), the
+    ``top`` largest (ties: the lower expert), and the softmax over those.  Returns int32 ``[T, top]``
+    experts and fp32 ``[T, top]`` weights, the largest logit first."""
+    _gpu(x, router, bias)
+    _need(x.dim() == 2 and x.stride(1) == 1, "x must be [T, dim] with unit column stride")
+    T, dim = x.shape
+    E = router.shape[0]
+    _need(router.dtype == torch.float32 and router.shape == (E, dim) and router.is_contiguous(),
+          "router must be contiguous float32 [E, dim]")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (E,) and bias.is_contiguous(), "bias must be float32 [E]")
+    _need(1 <= top <= E, f"top={top} must be between 1 and the {E} experts")
+    choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    weight = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    st = _lib.load("moe").fg_moe_route(_ptr(x), x.stride(0), _code(x), _ptr(router), _ptr(bias), T, dim, E, top,
+                                       _ptr(choice), _ptr(weight), _stream(x))
+    _check(st, "moe_route")
+    return choice, weight
+
+
+def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
+    """The most tiles of ``tile_rows`` rows that ``n_pairs`` rows spread over ``n_experts`` can make."""
+    return min(n_pairs, n_pairs // tile_rows + n_experts)
+
+
+def moe_sort(choice: torch.Tensor, n_experts: int, tile_rows: int):
+    """The (row, choice) pairs of ``choice [T, top]`` in the order of their experts, cut into tiles of
+    at most ``tile_rows`` rows of one expert, on the device.  Returns int32 ``sorted [T * top]`` (pair
+    ``t * top + j`` at each sorted place) and int32 ``tiles [max_tiles, 4]``: (expert, first sorted
+    place, rows, 0), rows = 0 for tiles that this step does not have."""
+    _gpu(choice)
+    _i32(choice, "choice")
+    n_pairs = choice.numel()
+    max_tiles = moe_max_tiles(n_pairs, n_experts, tile_rows)
+    sorted_ = torch.empty((n_pairs,), dtype=torch.int32, device=choice.device)
+    tiles = torch.empty((max_tiles, 4), dtype=torch.int32, device=choice.device)
+    st = _lib.load("moe").fg_moe_sort(_ptr(choice), n_pairs, n_experts, tile_rows, max_tiles, _ptr(sorted_), _ptr(tiles),
+                                      _stream(choice))
+    _check(st, "moe_sort")
+    return sorted_, tiles
+
+
+def _moe_mfma_ok(x: torch.Tensor, *weights: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and all(w.shape[2] % 8 == 0 and w.data_ptr() % 16 == 0 for w in weights))
+
+
+def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, sorted_: torch.Tensor, tiles: torch.Tensor,
+                top: int, tile_rows: int) -> torch.Tensor:
+    """``silu(x_t W_gate[e]^T) * (x_t W_up[e]^T)`` for every pair, in the sorted order: ``[T * top, hidden]``.
+    ``w_gate``, ``w_up``: ``[E, hidden, dim]`` of ``x``'s dtype.  bfloat16 with sizes in multiples of 8
+    runs on the matrix cores; everything else the fp32-FMA kernel (tiles of 16 rows only)."""
+    _gpu(x, w_gate, w_up, sorted_, tiles)
+    _need(x.dim() == 2 and x.stride(1) == 1 and w_gate.dim() == 3 and w_gate.shape == w_up.shape
+          and w_gate.shape[2] == x.shape[1] and w_gate.is_contiguous() and w_up.is_contiguous()
+          and w_gate.dtype == x.dtype == w_up.dtype, "x [T, dim], w_gate and w_up contiguous [E, hidden, dim] of x's dtype")
+    _i32(sorted_, "sorted", x.shape[0] * top)
+    _i32(tiles, "tiles")
+    _need(tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.data_ptr() % 16 == 0, "tiles must be [n, 4], 16-byte aligned")
+    hidden, dim = w_gate.shape[1], w_gate.shape[2]
+    mfma = _moe_mfma_ok(x, w_gate) and hidden % 8 == 0
+    _need(tile_rows in MOE_TILE_ROWS and (mfma or tile_rows == 16), "tile_rows does not fit the kernel")
+    act = torch.empty((sorted_.numel(), hidden), dtype=x.dtype, device=x.device)
+    st = _lib.load("moe").fg_moe_gate_up(_ptr(x), x.stride(0), _ptr(w_gate), _ptr(w_up), dim, _ptr(sorted_), _ptr(tiles),
+                                         tiles.shape[0], tile_rows, top, dim, hidden, _ptr(act), hidden, _code(x), int(mfma),
+                                         _stream(x))
+    _check(st, "moe_gate_up")
+    return act
+
+
+def moe_down(act: torch.Tensor, w_down: torch.Tensor, sorted_: torch.Tensor, tiles: torch.Tensor,
+             tile_rows: int) -> torch.Tensor:
+    """``act_p W_down[e]^T`` for every pair as fp32 ``[T * top, dim]``, row = pair (not the sorted order).
+    ``w_down``: ``[E, dim, hidden]`` of ``act``'s dtype."""
+    _gpu(act, w_down, sorted_, tiles)
+    _need(act.dim() == 2 and act.is_contiguous() and w_down.dim() == 3 and w_down.is_contiguous()
+          and w_down.shape[2] == act.shape[1] and w_down.dtype == act.dtype,
+          "act contiguous [pairs, hidden], w_down contiguous [E, dim, hidden] of act's dtype")
+    _i32(sorted_, "sorted", act.shape[0])
+    _i32(tiles, "tiles")
+    _need(tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.data_ptr() % 16 == 0, "tiles must be [n, 4], 16-byte aligned")
+    dim, hidden = w_down.shape[1], w_down.shape[2]
+    mfma = _moe_mfma_ok(act, w_down)
+    _need(tile_rows in MOE_TILE_ROWS and (mfma or tile_rows == 16), "tile_rows does not fit the kernel")
+    y = torch.empty((act.shape[0], dim), dtype=torch.float32, device=act.device)
+    st = _lib.load("moe").fg_moe_down(_ptr(act), hidden, _ptr(w_down), hidden, _ptr(sorted_), _ptr(tiles), tiles.shape[0],
+                                      tile_rows, dim, hidden, _ptr(y), _code(act), int(mfma), _stream(act))
+    _check(st, "moe_down")
+    return y
+
+
+def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 ``[1, T, dim]``: ``plus[t] + sum_j weight[t, j] * y[t * top + j]``, the weighted sum first, ``j``
+    ascending.  ``plus``: ``[T, dim]`` rows of any supported dtype, or None."""
+    _gpu(y, weight, plus)
+    T, top = weight.shape
+    _need(y.dtype == torch.float32 and y.dim() == 2 and y.shape[0] == T * top and y.is_contiguous()
+          and weight.dtype == torch.float32 and weight.is_contiguous(), "y float32 [T * top, dim], weight float32 [T, top]")
+    dim = y.shape[1]
+    if plus is not None:
+        _need(plus.shape == (T, dim) and plus.stride(1) == 1, "plus must be [T, dim]")
+    out = torch.empty((1, T, dim), dtype=torch.float32, device=y.device)
+    st = _lib.load("moe").fg_moe_combine(_ptr(y), _ptr(weight), _ptr(plus), plus.stride(0) if plus is not None else 0,
+                                         _code(plus) if plus is not None else F32, T, top, dim, _ptr(out), _stream(y))
+    _check(st, "moe_combine")
     return out

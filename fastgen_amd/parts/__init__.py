@@ -3,6 +3,7 @@ from .base import (
     TABLE_INT,
     VECTOR,
     FeedForward,
+    Injection,
     LayerStore,
     Mixer,
     Norm,
@@ -17,10 +18,10 @@ from .base import (
     registered_parts,
     unregister_part,
 )
-from . import attention, block, embedding, feed_forward, norm, position  # register the built-in parts
+from . import attention, block, embedding, feed_forward, injection, moe, norm, position  # register the built-in parts
 
 __all__ = [
-    "MATRIX", "TABLE_INT", "VECTOR", "FeedForward", "LayerStore", "Mixer", "Norm", "PagedNeed", "Part",
+    "MATRIX", "TABLE_INT", "VECTOR", "FeedForward", "Injection", "LayerStore", "Mixer", "Norm", "PagedNeed", "Part",
     "PositionEncoding", "StateNeed", "TensorSpec", "build_part", "place", "register_part",
     "registered_parts", "unregister_part",
 ]

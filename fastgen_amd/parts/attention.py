@@ -4,6 +4,13 @@ Per step (``fastgen/forward.py:421-472``): one product for q, k and v (the
 three projections are stored as one matrix), rotation of q and k and the
 write of k, v into the pages in one launch, attention of every new token
 over all cached keys of its request, output projection.
+
+Options beyond the reference's layer: ``value_from_key`` (there is no value
+projection: a token's value is its key as projected, before the rotation),
+``output_gate`` (the heads' outputs are multiplied by ``sigmoid(W_g x)`` before
+the output projection; ``W_g`` rides in the same product as q and k),
+``exact_weights`` (the softmax weights enter the product with the values in
+more than bfloat16's digits).
 """
 
 from __future__ import annotations
@@ -36,6 +43,9 @@ class Attention(Mixer):
                 f"{self.prefix}: head size {self.head_dim} is not supported: the cache and the attention"
                 " kernels work in chunks of 8 head dimensions, up to 512"
             )
+        self.value_from_key = bool(o.get("value_from_key", False))
+        self.output_gate = bool(o.get("output_gate", False))
+        self.exact_weights = bool(o.get("exact_weights", False))
         self.position = build_part("position", o["position"])
         self.wqkv: Optional[StreamedMatrix] = None
         self.wo: Optional[StreamedMatrix] = None
@@ -43,18 +53,24 @@ class Attention(Mixer):
 
     def tensor_specs(self) -> List[TensorSpec]:
         q, kv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
-        return [
-            TensorSpec(self._name("q_proj.weight"), (q, self.dim)),
-            TensorSpec(self._name("k_proj.weight"), (kv, self.dim)),
-            TensorSpec(self._name("v_proj.weight"), (kv, self.dim)),
-            TensorSpec(self._name("o_proj.weight"), (self.dim, q)),
-        ]
+        specs = [TensorSpec(self._name("q_proj.weight"), (q, self.dim)),
+                 TensorSpec(self._name("k_proj.weight"), (kv, self.dim))]
+        if not self.value_from_key:
+            specs.append(TensorSpec(self._name("v_proj.weight"), (kv, self.dim)))
+        if self.output_gate:
+            specs.append(TensorSpec(self._name("gate_proj.weight"), (q, self.dim)))
+        return specs + [TensorSpec(self._name("o_proj.weight"), (self.dim, q))]
 
     def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
-        wq = self.position.arrange_rows(tensors[self._name("q_proj.weight")], self.n_heads)
-        wk = self.position.arrange_rows(tensors[self._name("k_proj.weight")], self.n_kv_heads)
-        wv = tensors[self._name("v_proj.weight")]
-        self.wqkv = streamed(place(torch.cat([wq, wk, wv], dim=0), MATRIX, dtype, device))
+        # one matrix for everything that reads the mixer's input: q, k, then v (if it has a projection
+        # of its own), then the output gate
+        mats = [self.position.arrange_rows(tensors[self._name("q_proj.weight")], self.n_heads),
+                self.position.arrange_rows(tensors[self._name("k_proj.weight")], self.n_kv_heads)]
+        if not self.value_from_key:
+            mats.append(tensors[self._name("v_proj.weight")])
+        if self.output_gate:
+            mats.append(tensors[self._name("gate_proj.weight")])
+        self.wqkv = streamed(place(torch.cat(mats, dim=0), MATRIX, dtype, device))
         self.wo = streamed(place(tensors[self._name("o_proj.weight")], MATRIX, dtype, device))
         self.freqs = self.position.frequencies_on(device)
 
@@ -67,6 +83,10 @@ class Attention(Mixer):
         to the residual stream and that norm into its kernel and return ``ScaledRows``."""
         group = ctx.groups[store.group]
         q_width = self.n_heads * self.head_dim
+        kv_width = self.n_kv_heads * self.head_dim
+        # columns of the product: q, k, v (or none: the values are the k columns), gate
+        v_col = q_width if self.value_from_key else q_width + kv_width
+        gate_col = v_col + kv_width
         table = None
         if self.freqs is not None:
             # sin and cos of the step's positions: computed by the first layer, shared by all layers
@@ -76,23 +96,32 @@ class Attention(Mixer):
             if table is None:
                 table = ctx.scratch[key] = ops.rope_table(ctx.positions, self.freqs)
         rows = x.rows if isinstance(x, ops.ScaledRows) else x
-        if not (store.owns and self.head_dim % 16 == 0 and skinny_ok(rows, self.wqkv)) and rows is not x:
+        fused = store.owns and self.head_dim % 16 == 0 and skinny_ok(rows, self.wqkv)
+        if not fused and rows is not x:
             x = x.materialize()
-        if store.owns and self.head_dim % 16 == 0 and skinny_ok(rows, self.wqkv):
+        if fused:
             # few rows (decode): rotation and cache write happen where the product is stored
             qkv = ops.gemm_skinny_qkv(x, self.wqkv.streaming, table, group.slots, store.k_pages, store.v_pages, self.n_heads,
-                                      self.n_kv_heads, self.head_dim, self.position.rotary_dim)
+                                      self.n_kv_heads, self.head_dim, self.position.rotary_dim,
+                                      value_from_key=self.value_from_key, gate=self.output_gate)
+            gate = qkv[:, q_width:] if self.output_gate else None  # sigmoid applied where it was stored
+            gate_done = True
         else:
-            # an entry that reads another entry's cache needs its queries only
-            qkv = linear(x, self.wqkv if store.owns else self.wqkv.first_rows(q_width))
+            # an entry that reads another entry's cache needs its queries only (and its gate)
+            own_rows = self.wqkv if store.owns or self.output_gate else self.wqkv.first_rows(q_width)
+            qkv = linear(x, own_rows)
             ops.rope_kv_write(
                 qkv, ctx.positions, self.freqs, group.slots, store.k_pages, store.v_pages,
                 self.n_heads, self.n_kv_heads, self.head_dim, self.position.rotary_dim, write_kv=store.owns,
-                table=table,
+                table=table, v_col=v_col,
             )
+            gate = qkv[:, gate_col:] if self.output_gate else None
+            gate_done = False
         out = torch.empty((rows.shape[0], q_width), dtype=rows.dtype, device=rows.device)
         ops.paged_attention(qkv, out, store.k_pages, store.v_pages, group, ctx, self.n_heads, self.scale,
-                            self.window or 0)
+                            self.window or 0, exact_weights=self.exact_weights)
+        if gate is not None:
+            ops.gate_mul(out, gate, sigmoid=not gate_done)
         return linear(out, self.wo, partials_ok=True, residual=then)
 
 

@@ -104,6 +104,11 @@ class Part:
         self.prefix = spec.prefix
 
     def _name(self, suffix: str) -> str:
+        """The checkpoint's name of the part's tensor ``suffix``: the prefix and the suffix, or what
+        the spec's ``names`` option puts in the suffix's place (an empty string: the prefix alone)."""
+        suffix = self.spec.options.get("names", {}).get(suffix, suffix)
+        if not suffix:
+            return self.prefix
         return f"{self.prefix}.{suffix}" if self.prefix else suffix
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -155,6 +160,21 @@ class Norm(Part):
         raise NotImplementedError
 
 
+class Injection(Part):
+    """Something added to the residual stream between two layers, named by a run entry.
+
+    ``forward(h, pending, embedded, index)`` adds ``pending`` (what the layer before left to be
+    added, or None) and its own rows to the fp32 stream ``h`` in place.  ``embedded`` is the
+    embedding's output of this step (kept only if ``needs_embedding``), ``index`` the second number
+    of the entry's ``inject`` (which pass of a loop this is)."""
+
+    needs_embedding = False
+
+    def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], embedded: Optional[torch.Tensor],
+                index: int) -> None:
+        raise NotImplementedError
+
+
 class PositionEncoding(Part):
     """How positions enter a mixer.  A rotary scheme gives a frequency table,
     the number of leading head dimensions it rotates, and the row order in
@@ -185,6 +205,7 @@ _FREQUENCY_TABLES: Dict[Tuple[str, Tuple[float, ...]], torch.Tensor] = {}
 
 # -------------------------------------------------------------- registries
 _REGISTRIES: Dict[str, Dict[str, Callable[[PartSpec], Any]]] = {
+    "injection": {},
     "mixer": {},
     "feed_forward": {},
     "norm": {},

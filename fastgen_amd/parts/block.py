@@ -7,6 +7,7 @@ from typing import Any, Optional
 
 import torch
 
+from ..kernels import ops
 from ..kernels.ops import ScaledRows
 from .base import FeedForward, LayerStore, Mixer, Norm, register_part
 
@@ -48,3 +49,33 @@ class PreNormBlock:
 
 
 register_part("arrangement", "pre_norm", lambda spec, *parts: PreNormBlock(*parts))
+
+
+class ParallelBlock:
+    """``x = norm(h); h += mixer(x) + ffn(x)``: one norm, both sublayers read its output, and their
+    sum (taken first, in fp32) goes to the residual stream.  A layer without a feed-forward adds its
+    mixer's output alone.  Like the other arrangements it leaves the addition to whatever norm
+    follows: it takes the layer before's output as ``pending`` and returns its own un-added.
+
+    A feed-forward that can take the mixer's output into its last kernel (``adds_to``) returns the
+    sum as fp32 ``[1, T, dim]``; any other feed-forward's rows are added by a kernel of their own.
+    """
+
+    folds_norms = False
+
+    def __init__(self, mixer: Mixer, ffn: Optional[FeedForward], mixer_norm: Norm, ffn_norm: Optional[Norm] = None) -> None:
+        if ffn_norm is not None:
+            raise ValueError("a parallel layer has one norm: its feed-forward reads the mixer's")
+        self.mixer, self.ffn, self.mixer_norm = mixer, ffn, mixer_norm
+
+    def forward(self, h: torch.Tensor, pending, ctx: Any, store: LayerStore):
+        x = self.mixer_norm.forward(h, pending, ctx.act_dtype)
+        mixed = self.mixer.forward(x, ctx, store)
+        if self.ffn is None:
+            return mixed
+        if getattr(self.ffn, "adds_to", False):
+            return self.ffn.forward(x, plus=mixed)
+        return ops.add_rows(mixed, self.ffn.forward(x))
+
+
+register_part("arrangement", "parallel", lambda spec, *parts: ParallelBlock(*parts))

@@ -12,13 +12,14 @@ from .base import MATRIX, Part, TensorSpec, place, register_part
 
 
 class Embedding(Part):
-    """``h[t] = table[token[t]]`` into the fp32 residual stream, no scaling
-    (``fastgen/forward.py:406-409``)."""
+    """``h[t] = table[token[t]] * scale`` into the fp32 residual stream; ``scale`` is 1 unless the
+    spec says otherwise (``fastgen/forward.py:406-409`` has none)."""
 
     def __init__(self, spec) -> None:
         super().__init__(spec)
         self.vocab_size = int(spec.options["vocab_size"])
         self.dim = int(spec.options["dim"])
+        self.scale = float(spec.options.get("scale", 1.0))
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -31,7 +32,7 @@ class Embedding(Part):
         """``ctx`` is the step's context: an embedding that adds something per position (learned or
         computed absolute positions) finds ``ctx.positions`` there; this one does not look at it."""
         h = torch.empty((tokens.numel(), self.dim), dtype=torch.float32, device=tokens.device)
-        return ops.embed(self.weight, tokens, h)
+        return ops.embed(self.weight, tokens, h, self.scale)
 
 
 class LMHead(Part):

@@ -1,0 +1,92 @@
+"""A routed feed-forward: a mixture of gated experts.
+
+Every row goes to the ``top`` experts whose router logits are the largest
+(``x W_r^T + b`` in fp32), weighted by the softmax over those logits alone; an
+expert is ``W_down (silu(W_gate x) * (W_up x))`` without biases, and the output
+is the weighted sum of the chosen experts' outputs, taken in fp32.  All of it
+runs on the device (``csrc/moe.hip``): which rows went where is never looked
+at on the host, so a step with this part can be recorded.
+"""
+
+from __future__ import annotations
+
+from typing import Any, List, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import MATRIX, VECTOR, FeedForward, TensorSpec, place, register_part
+
+
+class MoE(FeedForward):
+    adds_to = True  # ``forward(x, plus=rows)`` returns plus + its own output, as fp32 [1, T, dim]
+
+    def __init__(self, spec) -> None:
+        super().__init__(spec)
+        o = spec.options
+        self.dim = int(o["dim"])
+        self.hidden_dim = int(o["hidden_dim"])
+        self.n_experts = int(o["n_experts"])
+        self.top = int(o["top"])
+        if not 1 <= self.top <= self.n_experts:
+            raise ValueError(f"{self.prefix}: top={self.top} must be between 1 and n_experts={self.n_experts}")
+        self.router_bias = bool(o.get("router_bias", True))
+        self.router: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+        self.w_gate: Optional[torch.Tensor] = None  # [E, hidden (padded to 8), dim]
+        self.w_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None  # [E, dim, hidden (padded to 8)]
+
+    def _expert(self, e: int, which: str) -> str:
+        names = self.spec.options.get("names", {})
+        return self._name(f"{names.get('expert', 'experts.{}').format(e)}.{names.get(which, which)}")
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [TensorSpec(self._name("router.weight"), (self.n_experts, self.dim), MATRIX, ("normal", 0.3))]
+        if self.router_bias:
+            specs.append(TensorSpec(self._name("router.bias"), (self.n_experts,), VECTOR, ("normal", 0.3)))
+        for e in range(self.n_experts):
+            specs += [TensorSpec(self._expert(e, "gate_proj.weight"), (self.hidden_dim, self.dim)),
+                      TensorSpec(self._expert(e, "up_proj.weight"), (self.hidden_dim, self.dim)),
+                      TensorSpec(self._expert(e, "down_proj.weight"), (self.dim, self.hidden_dim))]
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
+        # the router's logits are fp32 whatever the model's dtype is
+        self.router = tensors[self._name("router.weight")].to(device=device, dtype=torch.float32).contiguous()
+        if self.router_bias:
+            self.bias = tensors[self._name("router.bias")].to(device=device, dtype=torch.float32).contiguous()
+        gate = torch.stack([tensors[self._expert(e, "gate_proj.weight")] for e in range(self.n_experts)])
+        up = torch.stack([tensors[self._expert(e, "up_proj.weight")] for e in range(self.n_experts)])
+        down = torch.stack([tensors[self._expert(e, "down_proj.weight")] for e in range(self.n_experts)])
+        pad = -self.hidden_dim % 8
+        if pad:
+            # the matrix-core kernels read k in chunks of 8: channels of zero weights are added, whose
+            # activation silu(0) * 0 = 0 meets zero columns of the down projection
+            gate = torch.cat([gate, gate.new_zeros(self.n_experts, pad, self.dim)], dim=1)
+            up = torch.cat([up, up.new_zeros(self.n_experts, pad, self.dim)], dim=1)
+            down = torch.cat([down, down.new_zeros(self.n_experts, self.dim, pad)], dim=2)
+        self.w_gate = place(gate, MATRIX, dtype, device)
+        self.w_up = place(up, MATRIX, dtype, device)
+        self.w_down = place(down, MATRIX, dtype, device)
+
+    def tile_rows(self, n_rows: int) -> int:
+        """Rows of one expert a tile holds: 16, or more where the experts get so many rows each that
+        their matrices would otherwise be read many times over (the matrix-core kernels only)."""
+        if self.w_gate.dtype != torch.bfloat16 or self.dim % 8:
+            return 16
+        per_expert = n_rows * self.top / self.n_experts
+        return 64 if per_expert >= 48 else 32 if per_expert >= 24 else 16
+
+    def forward(self, x: torch.Tensor, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """fp32 ``[1, T, dim]``: the experts' weighted sum (plus ``plus``, rows that go to the
+        residual stream with it), for a norm to add."""
+        tile_rows = self.tile_rows(x.shape[0])
+        choice, weight = ops.moe_route(x, self.router, self.bias, self.top)
+        sorted_, tiles = ops.moe_sort(choice, self.n_experts, tile_rows)
+        act = ops.moe_gate_up(x, self.w_gate, self.w_up, sorted_, tiles, self.top, tile_rows)
+        y = ops.moe_down(act, self.w_down, sorted_, tiles, tile_rows)
+        return ops.moe_combine(y, weight, plus)
+
+
+register_part("feed_forward", "moe", MoE)

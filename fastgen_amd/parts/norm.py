@@ -11,19 +11,24 @@ from .base import VECTOR, Norm, TensorSpec, place, register_part
 
 
 class RMSNorm(Norm):
-    """``y = x * rsqrt(mean(x^2) + eps) * weight`` in fp32, one rounding."""
+    """``y = x * rsqrt(mean(x^2) + eps) * weight`` in fp32, one rounding.  With the option
+    ``unit_offset`` the checkpoint stores the weight around zero and ``1 + w`` is what multiplies
+    (kept in fp32: the sum has more digits than bfloat16 holds)."""
 
     def __init__(self, spec) -> None:
         super().__init__(spec)
         self.dim = int(spec.options["dim"])
         self.eps = float(spec.options["eps"])
+        self.unit_offset = bool(spec.options.get("unit_offset", False))
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self._name("weight"), (self.dim,), VECTOR, ("one_plus_normal", 0.01))]
+        init = ("normal", 0.1) if self.unit_offset else ("one_plus_normal", 0.01)
+        return [TensorSpec(self._name("weight"), (self.dim,), VECTOR, init)]
 
     def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
-        self.weight = place(tensors[self._name("weight")], VECTOR, dtype, device)
+        w = tensors[self._name("weight")]
+        self.weight = place(1.0 + w.to(torch.float32) if self.unit_offset else w, VECTOR, dtype, device)
 
     def fold_request(self, h: torch.Tensor):
         """(h, weight, eps): what a matrix product needs to fold the addition to the residual stream

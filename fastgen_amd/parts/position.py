@@ -31,6 +31,13 @@ class Rope(PositionEncoding):
         self.factor = float(o.get("factor", 1.0))
         self.low_freq_factor = float(o.get("low_freq_factor", 1.0))
         self.high_freq_factor = float(o.get("high_freq_factor", 1.0))
+        # linear scaling: every frequency is divided by this factor
+        self.linear_factor = float(o.get("linear_factor", 1.0))
+        # how the checkpoint pairs the rotated dimensions of a head: "half" (i with i + rotary_dim/2;
+        # its rows are permuted at load) or "interleaved" (2i with 2i+1: the kernels' own order)
+        self.pairing = o.get("pairing", "half")
+        if self.pairing not in ("half", "interleaved"):
+            raise ValueError(f"pairing={self.pairing!r} must be 'half' or 'interleaved'")
 
     def frequencies(self) -> Optional[torch.Tensor]:
         """fp32 ``[rotary_dim/2]``: ``1/theta^(2i/rotary_dim)``, then per
@@ -41,6 +48,8 @@ class Rope(PositionEncoding):
             return None
         exponents = torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim
         freqs = 1.0 / (self.theta ** exponents)
+        if self.linear_factor != 1.0:
+            freqs = freqs / self.linear_factor
         if not self.scaled:
             return freqs
         long_edge = self.original_context / self.low_freq_factor
@@ -64,7 +73,7 @@ class Rope(PositionEncoding):
         part of a head, stored row ``j`` (first half) goes to ``2j`` and row
         ``j + rotary_dim/2`` to ``2j+1``; rows past the rotary part stay."""
         hd, rd = self.head_dim, self.rotary_dim
-        if rd == 0:
+        if rd == 0 or self.pairing == "interleaved":
             return w
         idx = torch.arange(hd)
         # new row r of a head takes old row src[r]
