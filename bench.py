@@ -5,6 +5,7 @@
     python bench.py --workload serve        # continuous batching, see serve_workload()
     python bench.py --workload readme       # the load of the reference's README, see readme_workload()
     python bench.py --workload readme --shape 70b   # the same load at the 70B sizes, cache = the memory left
+    python bench.py --workload buderax      # the Buderax design beside the dense Llama at equal sizes
 
 The model has the layer sizes of Llama 3.1 8B (32 layers, hidden 4096, 32
 heads, 8 kv heads, head size 128, feed-forward 14336, vocabulary 128256,
@@ -181,6 +182,133 @@ def readme_workload(shape: str = "8b") -> int:
     return 0
 
 
+# Buderax at sizes that resemble a real model's layers; the dense Llama beside it has the same width, heads,
+# head size and number of layer runs, and a feed-forward as wide as the experts a token uses (top x ff).
+BUDERAX_SIZES = {
+    "w1024": dict(width=1024, heads=16, kv_heads=4, dim=64, experts=16, top=2, ff=512, layers=6,
+                  loop=dict(start=2, stop=4, times=2), vocab=32000),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=32, top=4, ff=768, layers=8, loop=None, vocab=32000),
+}
+
+
+def _buderax_configs(z: dict):
+    mixer = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5,
+                 rot=dict(base=500000.0, dims=z["dim"], scaling=dict(factor=4.0)))
+    mlp = dict(kind="moe", router=dict(experts=z["experts"], top=z["top"]), expert=dict(ff=z["ff"]))
+    new = dict(architecture="Buderax", width=z["width"], vocab=z["vocab"], embedding=dict(scale=2.0), norm=dict(eps=1e-6),
+               layers=[dict(type="attention", mixer=mixer, mlp=mlp) for _ in range(z["layers"])])
+    runs = z["layers"]
+    if z["loop"]:
+        new["loop"] = z["loop"]
+        runs += (z["loop"]["stop"] - z["loop"]["start"]) * (z["loop"]["times"] - 1)
+    dense = dict(architectures=["LlamaForCausalLM"], hidden_size=z["width"], intermediate_size=z["top"] * z["ff"],
+                 num_hidden_layers=runs, num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"],
+                 rms_norm_eps=1e-6, vocab_size=z["vocab"], rope_theta=500000.0, rope_scaling=None,
+                 tie_word_embeddings=False, max_position_embeddings=131072)
+    return new, dense, runs
+
+
+def _time(fn, repeats: int = 20) -> float:
+    """Seconds of one call: the best of ``repeats`` after three unmeasured ones."""
+    import torch
+
+    for _ in range(3):
+        fn()
+    best = float("inf")
+    for _ in range(repeats):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        best = min(best, a.elapsed_time(b) * 1e-3)
+    return best
+
+
+def _buderax_kernels(z: dict, rows: int) -> dict:
+    """The routed feed-forward's kernels at ``rows`` tokens beside the dense feed-forward's products with
+    the same rows and as many channels a token (top x ff): seconds, and the share of the roofline that
+    bounds them (matrix cores for many rows, memory for few: bytes = the matrices read once; of the
+    experts, those that the rows can reach)."""
+    import torch
+
+    from fastgen_amd.kernels import ops
+    from fastgen_amd.kernels.linear import linear
+
+    D, E, top, F = z["width"], z["experts"], z["top"], z["ff"]
+    g = torch.Generator(device="cuda").manual_seed(rows)
+    rnd = lambda *shape: (torch.randn(*shape, generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+    x = rnd(rows, D) * 20
+    router, bias = rnd(E, D).float(), rnd(E).float()
+    wg, wu, wd = rnd(E, F, D), rnd(E, F, D), rnd(E, D, F)
+    per_expert = rows * top / E
+    tile_rows = 64 if per_expert >= 48 else 32 if per_expert >= 24 else 16
+    choice, weight = ops.moe_route(x, router, bias, top)
+    sorted_, tiles = ops.moe_sort(choice, E, tile_rows)
+    act = ops.moe_gate_up(x, wg, wu, sorted_, tiles, top, tile_rows)
+    y = ops.moe_down(act, wd, sorted_, tiles, tile_rows)
+    dense_gu = ops.interleave_gate_up(rnd(top * F, D), rnd(top * F, D))
+    dense_d = rnd(D, top * F)
+    dense_act = linear(x, dense_gu, epilogue="silu_mul")
+    reached = min(E, rows * top)
+    flops_gu, flops_d = 2 * rows * top * 2 * F * D, 2 * rows * top * F * D
+    out = {}
+    for name, fn, flops, nbytes in (
+        ("moe_route", lambda: ops.moe_route(x, router, bias, top), 2 * rows * E * D, E * D * 4 + rows * D * 2),
+        ("moe_sort", lambda: ops.moe_sort(choice, E, tile_rows), 0, rows * top * 8),
+        ("moe_gate_up", lambda: ops.moe_gate_up(x, wg, wu, sorted_, tiles, top, tile_rows), flops_gu, reached * 2 * F * D * 2),
+        ("dense_gate_up", lambda: linear(x, dense_gu, epilogue="silu_mul"), flops_gu, top * 2 * F * D * 2),
+        ("moe_down", lambda: ops.moe_down(act, wd, sorted_, tiles, tile_rows), flops_d, reached * F * D * 2),
+        ("dense_down", lambda: linear(dense_act, dense_d), flops_d, top * F * D * 2),
+        ("moe_combine", lambda: ops.moe_combine(y, weight, None), 0, rows * top * D * 4 + rows * D * 4),
+    ):
+        t = _time(fn)
+        out[name] = {"us": round(t * 1e6, 1), "mfma_frac": round(flops / t / PEAK_FLOPS["bf16"], 4),
+                     "hbm_frac": round(nbytes / t / PEAK_HBM, 4)}
+    return out
+
+
+def buderax_workload(prefill_tokens: int = 2048, batch: int = 8, context: int = 1024, steps: int = 32, warmup: int = 8) -> int:
+    """Prefill and decode throughput of Buderax models with random bfloat16 weights beside dense Llama
+    models of equal sizes, and the routed feed-forward's kernels beside the dense feed-forward's.  One JSON line."""
+    import torch
+
+    from fastgen_amd.engine import Engine
+
+    results = {}
+    for name, z in BUDERAX_SIZES.items():
+        new, dense, runs = _buderax_configs(z)
+        row = {"layer_runs": runs}
+        for label, cfg in (("buderax", new), ("llama", dense)):
+            engine = Engine.from_config(cfg, seed=5, dtype=torch.bfloat16, page_size=PAGE,
+                                        max_tokens=max(batch * (context + 256), prefill_tokens + PAGE), max_batch=batch,
+                                        max_step_tokens=prefill_tokens)
+            g = torch.Generator().manual_seed(0)
+            prompt = lambda n: torch.randint(0, z["vocab"], (n,), generator=g).tolist()
+            pre = min(engine.time_prefill(prompt(prefill_tokens), repeats=5))
+            dt = engine.time_decode([prompt(context) for _ in range(batch)], steps=steps, warmup=warmup)
+            row[label] = {"prefill_tok_s": round(prefill_tokens / pre, 1), "prefill_ms": round(pre * 1e3, 3),
+                          "decode_tok_s": round(batch * steps / dt, 1), "decode_ms_per_step": round(dt / steps * 1e3, 4),
+                          "weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
+            print(f"[bench] {name} {label}: {row[label]}", file=sys.stderr, flush=True)
+            del engine
+            torch.cuda.empty_cache()
+        row["kernels_prefill"] = _buderax_kernels(z, prefill_tokens)
+        row["kernels_decode"] = _buderax_kernels(z, batch)
+        print(f"[bench] {name} kernels: {row['kernels_prefill']} {row['kernels_decode']}", file=sys.stderr, flush=True)
+        results[name] = row
+    first = results[next(iter(results))]
+    print(json.dumps({
+        "metric": "Buderax beside the dense Llama at equal sizes: prefill and decode tok/s", "unit": "tokens/s",
+        "value": first["buderax"]["decode_tok_s"], "n_gpus": 1, "steps": steps, "warmup": warmup, "higher_is_better": True,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"prefill_tokens": prefill_tokens, "decode_batch": batch, "decode_context": context, "page_size": PAGE,
+                   "sizes": BUDERAX_SIZES},
+        "results": results,
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -198,9 +326,10 @@ def main() -> int:
                          " 2,048); more are fed untimed, in portions")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
-    ap.add_argument("--workload", choices=["decode", "serve", "readme"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "serve", "readme", "buderax"], default="decode",
                     help="decode (default): the step benchmark; serve: continuous batching of 256 requests; "
-                         "readme: the load of the reference's README")
+                         "readme: the load of the reference's README; buderax: the Buderax design beside the dense "
+                         "Llama at equal sizes")
     ap.add_argument("--step-budget", type=int, default=2048, help="tokens a step of the serve workload")
     ap.add_argument("--show-choices", action="store_true",
                     help="print (stderr) which kernel the run's measurements chose for each matrix product")
@@ -212,6 +341,8 @@ def main() -> int:
         return serve_workload(step_budget=a.step_budget, shape=a.shape or "3b")
     if a.workload == "readme":
         return readme_workload(a.shape or "8b")
+    if a.workload == "buderax":
+        return buderax_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
     a.shape = a.shape or "8b"
 
     import torch

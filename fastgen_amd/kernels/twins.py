@@ -21,10 +21,41 @@ from ..cache.layout import store_k, store_v, unpack_k, unpack_v
 from .ops import PackedWeight, ScaledRows
 
 
-def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """``out[t] = table[tokens[t]]`` as fp32."""
-    out.copy_(table[tokens.long()].float())
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """``out[t] = table[tokens[t]] * scale`` as fp32."""
+    out.copy_(table[tokens.long()].float() * scale)
     return out
+
+
+def _added(delta: Optional[torch.Tensor]):
+    """What a ``delta`` argument adds, in order: rows ``[T, dim]``, or fp32 partial sums ``[S, T, dim]``."""
+    if delta is None:
+        return []
+    return [delta[s] for s in range(delta.shape[0])] if delta.dim() == 3 else [delta.float()]
+
+
+def stream_add(h: torch.Tensor, delta: Optional[torch.Tensor], again: Optional[torch.Tensor],
+               row: Optional[torch.Tensor]) -> torch.Tensor:
+    """``h = ((h + delta) + again) + row`` in place, fp32, in that order; each term may be None."""
+    for d in _added(delta):
+        h += d
+    if again is not None:
+        h += again
+    if row is not None:
+        h += row[None, :]
+    return h
+
+
+def add_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``a + b`` as fp32 ``[1, T, dim]``."""
+    return (a.float() + b.float())[None]
+
+
+def gate_mul(x: torch.Tensor, gate: torch.Tensor, sigmoid: bool = True) -> torch.Tensor:
+    """``x *= sigmoid(gate)`` (or ``gate`` itself) over the first ``x.shape[1]`` columns of ``gate``, in place."""
+    g = gate[:, : x.shape[1]].float()
+    x.copy_((x.float() * (torch.sigmoid(g) if sigmoid else g)).to(x.dtype))
+    return x
 
 
 def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
@@ -105,9 +136,11 @@ def _write_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, slots: torch.Tens
 
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[torch.Tensor], slots: torch.Tensor,
                   k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
-                  rotary_dim: int, write_kv: bool = True, table: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  rotary_dim: int, write_kv: bool = True, table: Optional[torch.Tensor] = None,
+                  v_col: Optional[int] = None) -> torch.Tensor:
     """``qkv [T, >= H*hd (+ 2*KV*hd)]``: q is rotated in place; k is rotated and, with v, written into the
-    pages (``fastgen/kernels/rope.py:56-89``, ``paged_memcpy.py:57-76``)."""
+    pages (``fastgen/kernels/rope.py:56-89``, ``paged_memcpy.py:57-76``).  The values are the columns from
+    ``v_col`` on (default: behind the keys; at the keys' own columns a value is its key before the rotation)."""
     T = qkv.shape[0]
     if rotary_dim and table is None:
         table = rope_table(positions, freqs)
@@ -116,7 +149,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[to
     qkv[:, :q_cols] = q.reshape(T, q_cols).to(qkv.dtype)
     if write_kv:
         k = _rotate(qkv[:, q_cols : q_cols + kv_cols].float().view(T, n_kv, head_dim), table, rotary_dim)
-        v = qkv[:, q_cols + kv_cols : q_cols + 2 * kv_cols].float().view(T, n_kv, head_dim)
+        v_col = q_cols + kv_cols if v_col is None else v_col
+        v = qkv[:, v_col : v_col + kv_cols].float().view(T, n_kv, head_dim)
         _write_pages(k_pages, v_pages, slots, k, v)
     return qkv
 
@@ -152,9 +186,10 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
                          plan=None, max_chunks=None, min_tiles: int = 4, max_rows: int = 16,
-                         tile_rows=None) -> torch.Tensor:
+                         tile_rows=None, exact_weights: bool = False) -> torch.Tensor:
     """The same attention for tokens listed as items (sequence, first flat token, tokens, position of the
-    first token).  How the kernels cut the work (``plan`` and what follows it) does not change the result."""
+    first token).  How the kernels cut the work (``plan`` and what follows it) does not change the result;
+    ``exact_weights`` only says how many digits of the softmax weights the kernel keeps (here: all)."""
     seq_of_token = torch.zeros(q.shape[0], dtype=torch.int32)
     positions = torch.zeros(q.shape[0], dtype=torch.int32)
     for items in (small_items, big_items):
@@ -168,7 +203,8 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
 
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
-                    group, ctx, n_heads: int, scale: float, window: int = 0) -> torch.Tensor:
+                    group, ctx, n_heads: int, scale: float, window: int = 0,
+                    exact_weights: bool = False) -> torch.Tensor:
     """Attention of one step: the block table from the layer's cache group, sequences and positions of the
     tokens from the step's context."""
     return paged_attention_general(q, out, k_pages, v_pages, group.block_table, ctx.seq_of_token, ctx.positions,
@@ -259,16 +295,88 @@ def gemm_skinny_residual(x, w, h: torch.Tensor, norm_weight: torch.Tensor, eps: 
 
 
 def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor, k_pages: torch.Tensor,
-                    v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rotary_dim: int) -> torch.Tensor:
+                    v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rotary_dim: int,
+                    value_from_key: bool = False, gate: bool = False) -> torch.Tensor:
     """The q, k, v projections with :func:`rope_kv_write` on the fp32 sums: returns the rotated queries in
-    bfloat16; the rotated keys and the values go into the pages."""
+    bfloat16; the rotated keys and the values go into the pages.  ``value_from_key``: there are no v rows,
+    the values are the keys before the rotation.  ``gate``: ``H * hd`` more rows, whose sigmoid is returned
+    behind the queries."""
     qkv = _rows(x) @ _matrix(wqkv).T
     T, q_cols, kv_cols = qkv.shape[0], n_heads * head_dim, n_kv * head_dim
     q = _rotate(qkv[:, :q_cols].view(T, n_heads, head_dim), table, rotary_dim)
-    k = _rotate(qkv[:, q_cols : q_cols + kv_cols].view(T, n_kv, head_dim), table, rotary_dim)
-    v = qkv[:, q_cols + kv_cols :].view(T, n_kv, head_dim)
+    k_raw = qkv[:, q_cols : q_cols + kv_cols].view(T, n_kv, head_dim)
+    k = _rotate(k_raw, table, rotary_dim)
+    v_end = q_cols + kv_cols if value_from_key else q_cols + 2 * kv_cols
+    v = k_raw if value_from_key else qkv[:, q_cols + kv_cols : v_end].view(T, n_kv, head_dim)
     _write_pages(k_pages, v_pages, slots, k, v)
-    return q.reshape(T, q_cols).to(torch.bfloat16)
+    out = q.reshape(T, q_cols)
+    if gate:
+        out = torch.cat([out, torch.sigmoid(qkv[:, v_end : v_end + q_cols])], dim=1)
+    return out.to(torch.bfloat16)
+
+
+# ------------------------------------------------------------- routed experts
+def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """The ``top`` experts with the largest fp32 logits ``x router^T + bias`` (largest first; of equal
+    logits the lower expert) and the softmax over those logits alone."""
+    z = x.float() @ router.T + (bias if bias is not None else 0.0)
+    val, idx = torch.sort(z, dim=-1, descending=True, stable=True)
+    return idx[:, :top].to(torch.int32), torch.softmax(val[:, :top], dim=-1)
+
+
+def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
+    return min(n_pairs, n_pairs // tile_rows + n_experts)
+
+
+def moe_sort(choice: torch.Tensor, n_experts: int, tile_rows: int):
+    """The pairs (row, choice) in the order of their experts (within an expert in any order; here:
+    ascending) and the tiles (expert, first sorted place, rows, 0) of at most ``tile_rows`` rows;
+    tiles that do not exist have zero rows."""
+    flat = choice.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    tiles = torch.zeros((moe_max_tiles(flat.numel(), n_experts, tile_rows), 4), dtype=torch.int32, device=choice.device)
+    at, first = 0, 0
+    for e, c in enumerate(torch.bincount(flat, minlength=n_experts).tolist()):
+        for r in range(0, c, tile_rows):
+            tiles[at] = torch.tensor([e, first + r, min(tile_rows, c - r), 0], dtype=torch.int32)
+            at += 1
+        first += c
+    return order.to(torch.int32), tiles
+
+
+def _expert_of_place(sorted_: torch.Tensor, tiles: torch.Tensor) -> torch.Tensor:
+    expert = torch.zeros(sorted_.numel(), dtype=torch.long, device=sorted_.device)
+    for e, first, rows, _ in tiles.tolist():
+        expert[first : first + rows] = e
+    return expert
+
+
+def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, sorted_: torch.Tensor, tiles: torch.Tensor,
+                top: int, tile_rows: int) -> torch.Tensor:
+    """``silu(x_t w_gate[e]^T) * (x_t w_up[e]^T)`` for the pair at every sorted place, ``e`` its expert."""
+    expert = _expert_of_place(sorted_, tiles)
+    rows = x[sorted_.long() // top].float()
+    g = torch.einsum("pk,pfk->pf", rows, w_gate[expert].float())
+    u = torch.einsum("pk,pfk->pf", rows, w_up[expert].float())
+    return (g * torch.sigmoid(g) * u).to(x.dtype)
+
+
+def moe_down(act: torch.Tensor, w_down: torch.Tensor, sorted_: torch.Tensor, tiles: torch.Tensor,
+             tile_rows: int) -> torch.Tensor:
+    """fp32 ``y[pair] = act[place of pair] w_down[e]^T``."""
+    expert = _expert_of_place(sorted_, tiles)
+    y = torch.empty((act.shape[0], w_down.shape[1]), dtype=torch.float32, device=act.device)
+    y[sorted_.long()] = torch.einsum("pf,pdf->pd", act.float(), w_down[expert].float())
+    return y
+
+
+def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 ``[1, T, dim]``: ``plus[t] + sum_j weight[t, j] * y[t * top + j]``."""
+    T, top = weight.shape
+    out = (weight[:, :, None] * y.view(T, top, -1)).sum(1)
+    if plus is not None:
+        out = out + plus.float()
+    return out[None]
 
 
 def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,

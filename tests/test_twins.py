@@ -23,7 +23,8 @@ from plain_llama import plain_attention, plain_rmsnorm, plain_rope_interleaved, 
 # functions of ops that launch a kernel (the others plan work, build arguments or pick a kernel)
 KERNEL_OPS = ["embed", "add_rmsnorm", "rmsnorm", "silu_mul", "rope_table", "rope_kv_write", "paged_attention_general",
               "paged_attention_mfma", "paged_attention", "gemm_nt", "scale_rows", "gemm_skinny_residual", "gemm_skinny",
-              "gemm_skinny_qkv", "gemm_tiled", "sample", "logprob"]
+              "gemm_skinny_qkv", "gemm_tiled", "sample", "logprob", "stream_add", "add_rows", "gate_mul", "moe_route",
+              "moe_sort", "moe_gate_up", "moe_down", "moe_combine"]
 
 
 @pytest.mark.parametrize("name", KERNEL_OPS + ["interleave_gate_up"])
@@ -386,3 +387,111 @@ def test_sample_and_logprob_twins(ops):
     tokens = torch.randint(0, 1003, (6,), dtype=torch.int32)
     _both("logprob", lambda: (logits, tokens), lambda g, w, *_: torch.testing.assert_close(g.cpu(), w, rtol=1e-5, atol=1e-5),
           ops)
+
+
+# ------------------------------------------- kernels of the gated attention and of the routed experts
+@gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_stream_add_add_rows_gate_mul_and_scaled_embed_twins(ops, dtype):
+    torch.manual_seed(3)
+    T, D = 9, 200
+    for delta in (None, torch.randn(T, D).to(dtype), torch.randn(3, T, D)):
+        for again in (None, torch.randn(T, D)):
+            make = lambda: (torch.randn(T, D), delta, again, torch.randn(D))
+            _both("stream_add", make, lambda g, w, *_: torch.testing.assert_close(g.cpu(), w, rtol=1e-6, atol=1e-6), ops)
+    _both("add_rows", lambda: (torch.randn(T, D).to(dtype), torch.randn(T, D).to(dtype)),
+          lambda g, w, *_: torch.testing.assert_close(g.cpu(), w, rtol=1e-6, atol=1e-6), ops)
+    wide = torch.randn(T, 2 * D).to(dtype)
+    for sigmoid in (True, False):
+        args = (torch.randn(T, D).to(dtype), wide, sigmoid)
+        got = ops.gate_mul(args[0].cuda(), wide.cuda()[:, D // 2:], sigmoid)
+        _close(got, twins.gate_mul(args[0].clone(), wide[:, D // 2:], sigmoid), dtype)
+    make = lambda: (torch.randn(50, D).to(dtype), torch.randint(0, 50, (T,), dtype=torch.int32), torch.zeros(T, D), 2.5)
+    _both("embed", make, lambda g, w, *_: torch.testing.assert_close(g.cpu(), w), ops)
+
+
+@gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KV,hd,rot,P", [(6, 2, 48, 16, 16), (5, 5, 80, 80, 64)])
+def test_rope_kv_write_with_values_from_the_keys_twin(ops, dtype, H, KV, hd, rot, P):
+    torch.manual_seed(hd + 1)
+    T = 21
+    pos = torch.randint(0, 5000, (T,), dtype=torch.int32)
+    slots = torch.randperm(6 * P)[:T].to(torch.int32)
+    slots[7] = -1
+    freqs = 1.0 / 500000.0 ** (torch.arange(0, rot, 2).float() / rot) / 4.0
+    # rows of q, k and a gate: no v columns, the values are read from the k columns
+    make = lambda: (torch.randn(T, (2 * H + KV) * hd).to(dtype), pos, freqs, slots, torch.zeros(6, KV, P, hd).to(dtype),
+                    torch.zeros(6, KV, hd, P).to(dtype), H, KV, hd, rot, True, None, H * hd)
+
+    def compare(got, want, dev, cpu):
+        for i in (0, 4, 5):
+            _close(dev[i], cpu[i], dtype)
+        assert float(cpu[5].abs().max()) > 0
+    _both("rope_kv_write", make, compare, ops)
+
+
+@gpu
+@pytest.mark.parametrize("M,H,KV,hd,rot,P,K,from_key,gate", [(5, 6, 2, 48, 16, 16, 72, True, True),
+                                                          (16, 5, 1, 80, 80, 64, 520, True, False),
+                                                          (3, 4, 4, 32, 32, 32, 136, False, True)])
+def test_gemm_skinny_qkv_with_gate_and_values_from_the_keys_twin(ops, M, H, KV, hd, rot, P, K, from_key, gate):
+    torch.manual_seed(K + 1)
+    bf = torch.bfloat16
+    n_rows = (H + (1 if from_key else 2) * KV) * hd + (H * hd if gate else 0)
+    x, w = (torch.randn(M, K) / 4).to(bf), (torch.randn(n_rows, K) / 4).to(bf)
+    pos = torch.randint(0, 3000, (M,), dtype=torch.int32)
+    freqs = 1.0 / 10000.0 ** (torch.arange(0, rot, 2).float() / rot)
+    table = twins.rope_table(pos, freqs)
+    slots = torch.randperm(4 * P)[:M].to(torch.int32)
+    make = lambda: (x, w, table, slots, torch.zeros(4, KV, P, hd).to(bf), torch.zeros(4, KV, hd, P).to(bf), H, KV, hd, rot,
+                    from_key, gate)
+
+    def compare(got, want, dev, cpu):
+        assert got.shape == want.shape == (M, (2 if gate else 1) * H * hd)
+        _close(got, want, bf)
+        _close(dev[4], cpu[4], bf)
+        _close(dev[5], cpu[5], bf)
+    _both("gemm_skinny_qkv", make, compare, ops)
+    # the same through a packed copy of the matrix
+    packed = kernel_ops.pack_weight(w.cuda())
+    dev = [a.cuda() if isinstance(a, torch.Tensor) else a for a in make()]
+    dev[1] = packed
+    _close(ops.gemm_skinny_qkv(*dev), twins.gemm_skinny_qkv(*make()), bf)
+
+
+@gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,D,E,top,F,tile_rows", [(7, 72, 5, 2, 24, 16), (300, 136, 3, 2, 40, 64), (90, 64, 4, 4, 16, 32),
+                                                  (1, 40, 70, 3, 8, 16)])
+def test_routed_expert_kernels_twins(ops, dtype, T, D, E, top, F, tile_rows):
+    torch.manual_seed(T + E)
+    if dtype == torch.float32:
+        tile_rows = 16
+    x = torch.randn(T, D).to(dtype)
+    router, bias = torch.randn(E, D), torch.randn(E)
+    choice_w = {}
+
+    def keep(got, want, *_):
+        assert torch.equal(got[0].cpu(), want[0])
+        torch.testing.assert_close(got[1].cpu(), want[1], rtol=1e-5, atol=1e-6)
+        choice_w["c"], choice_w["w"] = want
+    _both("moe_route", lambda: (x, router, bias, top), keep, ops)
+    choice, weight = choice_w["c"], choice_w["w"]
+    sorted_d, tiles_d = ops.moe_sort(choice.cuda(), E, tile_rows)
+    sorted_c, tiles_c = twins.moe_sort(choice, E, tile_rows)
+    assert torch.equal(tiles_d.cpu(), tiles_c)
+    # within an expert the kernel's order is free: the same pairs at each expert's places
+    for e, first, rows, _ in tiles_c.tolist():
+        assert sorted(sorted_d.cpu()[first:first + rows].tolist()) == sorted(sorted_c[first:first + rows].tolist())
+    wg, wu, wd = (torch.randn(E, F, D) / 4).to(dtype), (torch.randn(E, F, D) / 4).to(dtype), (torch.randn(E, D, F) / 4).to(dtype)
+    act_d = ops.moe_gate_up(x.cuda(), wg.cuda(), wu.cuda(), sorted_d, tiles_d, top, tile_rows)
+    act_c = twins.moe_gate_up(x, wg, wu, sorted_d.cpu(), tiles_c, top, tile_rows)
+    _close(act_d, act_c, dtype)
+    y_d = ops.moe_down(act_d, wd.cuda(), sorted_d, tiles_d, tile_rows)
+    y_c = twins.moe_down(act_d.cpu(), wd, sorted_d.cpu(), tiles_c, tile_rows)
+    _close(y_d, y_c, dtype)
+    plus = torch.randn(T, D).to(dtype)
+    for p in (None, plus):
+        got = ops.moe_combine(y_d, weight.cuda(), p.cuda() if p is not None else None)
+        torch.testing.assert_close(got.cpu(), twins.moe_combine(y_d.cpu(), weight, p), rtol=1e-5, atol=1e-5)
