@@ -242,7 +242,7 @@ def _buderax_kernels(z: dict, rows: int) -> dict:
     router, bias = rnd(E, D).float(), rnd(E).float()
     wg, wu, wd = rnd(E, F, D), rnd(E, F, D), rnd(E, D, F)
     per_expert = rows * top / E
-    tile_rows = 64 if per_expert >= 48 else 32 if per_expert >= 24 else 16
+    tile_rows = next((r for r, least in ((256, 768), (128, 96), (64, 48), (32, 24)) if per_expert >= least), 16)
     choice, weight = ops.moe_route(x, router, bias, top)
     sorted_, tiles = ops.moe_sort(choice, E, tile_rows)
     act = ops.moe_gate_up(x, wg, wu, sorted_, tiles, top, tile_rows)

@@ -20,25 +20,60 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ------------------------------------------------------------------- route
-// One wave a token.  LDS per wave: n_experts logits, then `top` chosen values.
+// Logits: a wave computes ROUTE_EPW experts' logits of one token (the row of x is read once for them),
+// eight elements a lane and round; lanes' partial sums are added by the wave in a fixed order.
+#define ROUTE_EPW 4
 template <class T>
-__global__ __launch_bounds__(256) void moe_route_kernel(
+__global__ __launch_bounds__(256) void moe_logits_kernel(
     const T* __restrict__ x, int ldx, const float* __restrict__ wr, const float* __restrict__ bias,
-    int n_tokens, int dim, int n_experts, int top, int* __restrict__ choice, float* __restrict__ weight) {
+    int n_tokens, int dim, int n_experts, float* __restrict__ z) {
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int groups = (n_experts + ROUTE_EPW - 1) / ROUTE_EPW;
+  const long long item = (long long)blockIdx.x * 4 + wave;
+  if (item >= (long long)n_tokens * groups) return;
+  const int t = (int)(item / groups), e0 = (int)(item % groups) * ROUTE_EPW;
+  const T* xr = x + (size_t)t * ldx;
+  float s[ROUTE_EPW];
+#pragma unroll
+  for (int j = 0; j < ROUTE_EPW; ++j) s[j] = 0.f;
+  if (dim % 8 == 0 && ldx % 8 == 0) {
+    for (int k = lane * 8; k < dim; k += FG_WAVE * 8) {
+      float xv[8];
+      load8<T>(xr + k, xv);
+#pragma unroll
+      for (int j = 0; j < ROUTE_EPW; ++j) {
+        float wv[8];
+        load8<float>(wr + (size_t)min(e0 + j, n_experts - 1) * dim + k, wv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s[j] = fmaf(xv[i], wv[i], s[j]);
+      }
+    }
+  } else {
+    for (int k = lane; k < dim; k += FG_WAVE) {
+      const float xv = to_f<T>(xr[k]);
+#pragma unroll
+      for (int j = 0; j < ROUTE_EPW; ++j) s[j] = fmaf(xv, wr[(size_t)min(e0 + j, n_experts - 1) * dim + k], s[j]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < ROUTE_EPW; ++j) {
+    const float v = wave_sum(s[j]);
+    if (lane == 0 && e0 + j < n_experts) z[(size_t)t * n_experts + e0 + j] = v + (bias ? bias[e0 + j] : 0.f);
+  }
+}
+
+// The `top` largest logits of a token (ties: the lower expert) and the softmax over them: a wave a token.
+// LDS per wave: n_experts logits, then `top` chosen values.
+__global__ __launch_bounds__(256) void moe_topk_kernel(
+    const float* __restrict__ zg, int n_tokens, int n_experts, int top, int* __restrict__ choice,
+    float* __restrict__ weight) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int t_raw = blockIdx.x * 4 + wave;
-  const int t = min(t_raw, n_tokens - 1);  // a wave beyond the tokens computes the last one again and stores nothing
+  const int t = min(t_raw, n_tokens - 1);  // a wave beyond the tokens does the last one again and stores nothing
   float* z = lds + (size_t)wave * (n_experts + top);
   float* chosen = z + n_experts;
-  const T* xr = x + (size_t)t * ldx;
-  for (int e = 0; e < n_experts; ++e) {
-    const float* w = wr + (size_t)e * dim;
-    float s = 0.f;
-    for (int k = lane; k < dim; k += FG_WAVE) s = fmaf(to_f<T>(xr[k]), w[k], s);
-    s = wave_sum(s);
-    if (lane == 0) z[e] = s + (bias ? bias[e] : 0.f);
-  }
+  for (int e = lane; e < n_experts; e += FG_WAVE) z[e] = zg[(size_t)t * n_experts + e];
   __syncthreads();
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
@@ -70,21 +105,23 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
   }
 }
 
+// z: fp32 scratch [n_tokens, n_experts] for the logits
 extern "C" int fg_moe_route(const void* x, int ldx, int dtype, const float* wr, const float* bias, int n_tokens, int dim,
-                            int n_experts, int top, int* choice, float* weight, hipStream_t stream) {
+                            int n_experts, int top, float* z, int* choice, float* weight, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
-  if (dim <= 0 || ldx < dim || n_experts <= 0 || top < 1 || top > n_experts) return FG_ERR_ARG;
+  if (dim <= 0 || ldx < dim || n_experts <= 0 || top < 1 || top > n_experts || !z) return FG_ERR_ARG;
   const size_t lds = (size_t)4 * (n_experts + top) * sizeof(float);
   if (lds > 60000) return FG_ERR_ARG;
-  const int blocks = (n_tokens + 3) / 4;
+  const long long items = (long long)n_tokens * ((n_experts + ROUTE_EPW - 1) / ROUTE_EPW);
+  if ((items + 3) / 4 > 2147483647LL) return FG_ERR_ARG;
+  const unsigned blocks = (unsigned)((items + 3) / 4);
   if (dtype == FG_F32)
-    moe_route_kernel<float><<<blocks, 256, lds, stream>>>((const float*)x, ldx, wr, bias, n_tokens, dim, n_experts, top,
-                                                          choice, weight);
+    moe_logits_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, ldx, wr, bias, n_tokens, dim, n_experts, z);
   else if (dtype == FG_BF16)
-    moe_route_kernel<bf16_t><<<blocks, 256, lds, stream>>>((const bf16_t*)x, ldx, wr, bias, n_tokens, dim, n_experts,
-                                                           top, choice, weight);
+    moe_logits_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, wr, bias, n_tokens, dim, n_experts, z);
   else
     return FG_ERR_ARG;
+  moe_topk_kernel<<<(n_tokens + 3) / 4, 256, lds, stream>>>(z, n_tokens, n_experts, top, choice, weight);
   return fg_launch_status();
 }
 
@@ -316,8 +353,150 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
   }
 }
 
+// ------------------------------------------------------- large tiles through LDS
+// Many rows an expert (prompt steps): a workgroup owns a tile of up to 64 WM rows of one expert and 128
+// output columns, its WM x 2 waves 64 x 64 each; both operands go from memory straight into LDS
+// (global_load_lds) through a ring of NST stages of 32 k, as in gemm_tiled.hip, whose loop this is.  What
+// differs is where the rows come from and go to: the tile's rows of x are gathered by token (gate_up) or
+// are its sorted places (down), the matrix is the tile's expert's, and for gate_up its 16-row blocks are
+// made of 8 gate rows and the 8 up rows of the same channels as they are loaded (nothing is stored
+// interleaved), so that silu(gate) * up is applied to the accumulators.
+#define MT_GATE_UP 0
+#define MT_DOWN 1
+
+template <int N>
+__device__ __forceinline__ void moe_wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int WM, int NST, int EPI>
+__global__ __launch_bounds__(128 * WM) void moe_tiled_kernel(
+    const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w0, const bf16_t* __restrict__ w1, int ldw,
+    void* __restrict__ y, int ldy, const int* __restrict__ sorted, const int* __restrict__ tiles, int top,
+    int N /* rows of the matrix as the tile sees it: 2 * hidden (gate_up), dim (down) */, int K) {
+  constexpr int WN = 2, NW = WM * WN, WB = 4 * WN, XB = 4 * WM, NB = WB + XB, LPW = NB / NW, BLOCK = 16 * 32;
+  static_assert(NB % NW == 0 && NST >= 3 && LPW * (NST - 2) < 64, "blocks divide over the waves; loads fit the counter");
+  extern __shared__ __attribute__((aligned(16))) bf16_t ring[];  // [NST][NB][BLOCK]
+  const int4 tile = *(const int4*)(tiles + 4 * (size_t)blockIdx.y);
+  if (tile.z <= 0) return;  // (the whole workgroup)
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int wm = wave / WN, wn = wave % WN;
+  const int n_base = blockIdx.x * (64 * WN);
+  const int n_stages = (K + 31) / 32;
+
+  const bf16_t* src[LPW];
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) {
+    const int b = wave + NW * j;
+    if (b >= WB) {
+      const int pos = tile.y + min(16 * (b - WB) + r16, tile.z - 1);  // rows beyond the tile: its last row, not stored
+      src[j] = x + (size_t)(EPI == MT_GATE_UP ? sorted[pos] / top : pos) * ldx + 8 * g;
+    } else {
+      const int vr = min(n_base + 16 * b + r16, N - 1);
+      if (EPI == MT_GATE_UP)
+        src[j] = ((vr & 8) ? w1 : w0) + ((size_t)tile.x * (N >> 1) + ((vr >> 4) << 3) + (vr & 7)) * ldw + 8 * g;
+      else
+        src[j] = w0 + ((size_t)tile.x * N + vr) * ldw + 8 * g;
+    }
+  }
+  auto issue = [&](int s) {
+    const int k = 32 * min(s, n_stages - 1);
+    const int koff = k + 8 * g < K ? k : 0;  // a chunk beyond k: any readable one, zeroed at use
+    bf16_t* slot = ring + (size_t)(s % NST) * NB * BLOCK;
+#pragma unroll
+    for (int j = 0; j < LPW; ++j)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[j] + koff),
+                                       (__attribute__((address_space(3))) void*)(slot + (wave + NW * j) * BLOCK), 16, 0, 0);
+  };
+
+  f32x4 acc[4][4];  // [row block mb][column block nb]
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < NST - 1; ++s) issue(s);
+  for (int i = 0; i < n_stages; ++i) {
+    moe_wait_vmcnt<LPW*(NST - 2)>();  // this wave's loads of stage i have landed
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();  // everybody's have, and nobody reads stage i - 1 any more
+    asm volatile("" ::: "memory");
+    issue(i + NST - 1);
+    const bf16_t* st = ring + (size_t)(i % NST) * NB * BLOCK;
+    const bool in = 32 * i + 8 * g < K;
+    bf16x8 a[4], b[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      a[nb] = *(const bf16x8*)(st + (wn * 4 + nb) * BLOCK + lane * 8);
+      a[nb] = in ? a[nb] : moe_zero8();
+    }
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) b[mb] = *(const bf16x8*)(st + (WB + wm * 4 + mb) * BLOCK + lane * 8);
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nb], b[mb], acc[mb][nb], 0, 0, 0);
+  }
+  moe_wait_vmcnt<0>();  // the loads issued past the end land before the workgroup's LDS is given up
+
+  // acc[mb][nb][i]: the tile's row 64 wm + 16 mb + r16, matrix row n_base + 64 wn + 16 nb + 4 g + i
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    const int ml = 64 * wm + 16 * mb + r16;
+    const bool valid = ml < tile.z;
+    const int pos = tile.y + min(ml, tile.z - 1);
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      const int n0 = n_base + 64 * wn + 16 * nb;
+      if (EPI == MT_DOWN) {
+        const int n = n0 + 4 * g;
+        if (!valid) continue;
+        float* dst = (float*)y + (size_t)sorted[pos] * ldy + n;
+        if (n + 3 < N && (ldy & 3) == 0) {
+          *(f32x4*)dst = acc[mb][nb];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) dst[i] = acc[mb][nb][i];
+        }
+      } else {
+        // lane groups 0, 1 hold the gate rows 4 g + i of 8 channels, groups 2, 3 the up rows of the same channels
+        bf16x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float up = __shfl_xor(acc[mb][nb][i], 32, FG_WAVE);
+          const float gate = acc[mb][nb][i];
+          v[i] = (__bf16)(gate * __frcp_rn(1.f + __expf(-gate)) * up);
+        }
+        if (g < 2 && valid && n0 + 15 < N) *(bf16x4*)((bf16_t*)y + (size_t)pos * ldy + n0 / 2 + 4 * g) = v;
+      }
+    }
+  }
+}
+
+template <int WM, int EPI>
+static int launch_moe_tiled(const void* x, int ldx, const void* w0, const void* w1, int ldw, void* y, int ldy,
+                            const int* sorted, const int* tiles, int max_tiles, int top, int N, int K, hipStream_t stream) {
+  constexpr int NST = 4, lds = NST * 4 * (WM + 2) * 1024;
+  static bool raised = false;  // more than 64 KB of dynamic LDS has to be asked for once
+  auto kernel = moe_tiled_kernel<WM, NST, EPI>;
+  if (lds > 65536 && !raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return FG_ERR_LAUNCH;
+    raised = true;
+  }
+  if (max_tiles > 65535) return FG_ERR_ARG;
+  const dim3 grid((N + 127) / 128, max_tiles);
+  kernel<<<grid, 128 * WM, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w0, (const bf16_t*)w1, ldw, y, ldy, sorted,
+                                          tiles, top, N, K);
+  return fg_launch_status();
+}
+
 // x [T, dim] rows gathered by token; wg, wu [E, hidden, ldw], act [n_pairs, lda] in the sorted order.
-// mfma: bf16 with dim % 8 == 0, ldx % 8 == 0, ldw % 8 == 0 (16-byte loads); tile_rows = 16 * MB, MB in 1, 2, 4.
+// mfma: bf16 with dim % 8 == 0, ldx % 8 == 0, ldw % 8 == 0 (16-byte loads); tile_rows = 16 * MB, MB in 1, 2, 4,
+// or 128 / 256: the tiles that go through LDS.
 extern "C" int fg_moe_gate_up(const void* x, int ldx, const void* wg, const void* wu, int ldw, const int* sorted,
                               const int* tiles, int max_tiles, int tile_rows, int top, int dim, int hidden, void* act,
                               int lda, int dtype, int mfma, hipStream_t stream) {
@@ -325,6 +504,12 @@ extern "C" int fg_moe_gate_up(const void* x, int ldx, const void* wg, const void
   if (dim <= 0 || hidden <= 0 || top <= 0 || ldx < dim || ldw < dim || lda < hidden) return FG_ERR_ARG;
   if (mfma) {
     if (dtype != FG_BF16 || dim % 8 || ldx % 8 || ldw % 8 || lda % 4) return FG_ERR_ARG;
+    if (tile_rows == 128 || tile_rows == 256) {
+      if (hidden % 8 || dim < 32) return FG_ERR_ARG;  // (a lane's stand-in load reads the row's first 32 k)
+      return tile_rows == 128
+                 ? launch_moe_tiled<2, MT_GATE_UP>(x, ldx, wg, wu, ldw, act, lda, sorted, tiles, max_tiles, top, 2 * hidden, dim, stream)
+                 : launch_moe_tiled<4, MT_GATE_UP>(x, ldx, wg, wu, ldw, act, lda, sorted, tiles, max_tiles, top, 2 * hidden, dim, stream);
+    }
     const long long items = (long long)max_tiles * ((hidden + 15) / 16);
     const unsigned blocks = (unsigned)((items + 3) / 4);
 #define GO(MB)                                                                                                   \
@@ -360,6 +545,11 @@ extern "C" int fg_moe_down(const void* act, int lda, const void* wd, int ldw, co
   if (dim <= 0 || hidden <= 0 || lda < hidden || ldw < hidden) return FG_ERR_ARG;
   if (mfma) {
     if (dtype != FG_BF16 || hidden % 8 || lda % 8 || ldw % 8) return FG_ERR_ARG;
+    if ((tile_rows == 128 || tile_rows == 256) && hidden < 32) return FG_ERR_ARG;
+    if (tile_rows == 128 || tile_rows == 256)
+      return tile_rows == 128
+                 ? launch_moe_tiled<2, MT_DOWN>(act, lda, wd, nullptr, ldw, y, dim, sorted, tiles, max_tiles, 1, dim, hidden, stream)
+                 : launch_moe_tiled<4, MT_DOWN>(act, lda, wd, nullptr, ldw, y, dim, sorted, tiles, max_tiles, 1, dim, hidden, stream);
     const long long items = (long long)max_tiles * ((dim + 15) / 16);
     const unsigned blocks = (unsigned)((items + 3) / 4);
 #define GO(MB)                                                                                                      \
@@ -388,27 +578,35 @@ extern "C" int fg_moe_down(const void* act, int lda, const void* wd, int ldw, co
 
 // ----------------------------------------------------------------- combine
 // out[t] = plus[t] + sum_j weight[t][j] * y[t * top + j]: the weighted sum first, j ascending, all fp32.
+// plus: rows of the activation dtype, or (n_plus > 0) fp32 partial sums plus[p * plus_stride + t * ldp + d],
+// whose sum, in order, is what is added.
 template <class TP>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
-    const float* __restrict__ y, const float* __restrict__ weight, const TP* __restrict__ plus, int ldp, int top, int dim,
-    float* __restrict__ out) {
+    const float* __restrict__ y, const float* __restrict__ weight, const TP* __restrict__ plus, int ldp, int n_plus,
+    size_t plus_stride, int top, int dim, float* __restrict__ out) {
   const int t = blockIdx.x;
   for (int d = threadIdx.x; d < dim; d += 256) {
     float s = 0.f;
     for (int j = 0; j < top; ++j) s = fmaf(weight[(size_t)t * top + j], y[((size_t)t * top + j) * dim + d], s);
-    if (plus) s += to_f<TP>(plus[(size_t)t * ldp + d]);
+    if (plus) {
+      float m = to_f<TP>(plus[(size_t)t * ldp + d]);
+      for (int p = 1; p < n_plus; ++p) m += to_f<TP>(plus[p * plus_stride + (size_t)t * ldp + d]);
+      s = m + s;
+    }
     out[(size_t)t * dim + d] = s;
   }
 }
 
-extern "C" int fg_moe_combine(const float* y, const float* weight, const void* plus, int ldp, int plus_dtype,
-                              int n_tokens, int top, int dim, float* out, hipStream_t stream) {
+extern "C" int fg_moe_combine(const float* y, const float* weight, const void* plus, int ldp, int plus_dtype, int n_plus,
+                              long long plus_stride, int n_tokens, int top, int dim, float* out, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
-  if (top <= 0 || dim <= 0 || (plus && ldp < dim)) return FG_ERR_ARG;
+  if (top <= 0 || dim <= 0 || (plus && (ldp < dim || n_plus < 1)) || (n_plus > 1 && plus_dtype != FG_F32)) return FG_ERR_ARG;
   if (plus_dtype == FG_F32)
-    moe_combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weight, (const float*)plus, ldp, top, dim, out);
+    moe_combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weight, (const float*)plus, ldp, n_plus, (size_t)plus_stride,
+                                                            top, dim, out);
   else if (plus_dtype == FG_BF16)
-    moe_combine_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(y, weight, (const bf16_t*)plus, ldp, top, dim, out);
+    moe_combine_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(y, weight, (const bf16_t*)plus, ldp, n_plus,
+                                                             (size_t)plus_stride, top, dim, out);
   else
     return FG_ERR_ARG;
   return fg_launch_status();

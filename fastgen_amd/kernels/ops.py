@@ -891,7 +891,7 @@ def logprob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
 
 
 # ------------------------------------------------------------- routed experts
-MOE_TILE_ROWS = (16, 32, 64)  # rows of one expert that a tile of the matrix-core kernels holds
+MOE_TILE_ROWS = (16, 32, 64, 128, 256)  # rows of one expert that a tile of the matrix-core kernels holds (from 128: through LDS)
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
@@ -899,7 +899,7 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     ``top`` largest (ties: the lower expert), and the softmax over those.  Returns int32 ``[T, top]``
     experts and fp32 ``[T, top]`` weights, the largest logit first."""
     _gpu(x, router, bias)
-    _need(x.dim() == 2 and x.stride(1) == 1, "x must be [T, dim] with unit column stride")
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.data_ptr() % 16 == 0, "x must be [T, dim] with unit column stride")
     T, dim = x.shape
     E = router.shape[0]
     _need(router.dtype == torch.float32 and router.shape == (E, dim) and router.is_contiguous(),
@@ -909,8 +909,9 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     _need(1 <= top <= E, f"top={top} must be between 1 and the {E} experts")
     choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weight = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
     st = _lib.load("moe").fg_moe_route(_ptr(x), x.stride(0), _code(x), _ptr(router), _ptr(bias), T, dim, E, top,
-                                       _ptr(choice), _ptr(weight), _stream(x))
+                                       _ptr(logits), _ptr(choice), _ptr(weight), _stream(x))
     _check(st, "moe_route")
     return choice, weight
 
@@ -988,16 +989,23 @@ def moe_down(act: torch.Tensor, w_down: torch.Tensor, sorted_: torch.Tensor, til
 
 def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 ``[1, T, dim]``: ``plus[t] + sum_j weight[t, j] * y[t * top + j]``, the weighted sum first, ``j``
-    ascending.  ``plus``: ``[T, dim]`` rows of any supported dtype, or None."""
+    ascending.  ``plus``: ``[T, dim]`` rows of any supported dtype, fp32 ``[S, T, dim]`` partial sums (a
+    product whose k range was cut; summed in order), or None."""
     _gpu(y, weight, plus)
     T, top = weight.shape
     _need(y.dtype == torch.float32 and y.dim() == 2 and y.shape[0] == T * top and y.is_contiguous()
           and weight.dtype == torch.float32 and weight.is_contiguous(), "y float32 [T * top, dim], weight float32 [T, top]")
     dim = y.shape[1]
-    if plus is not None:
+    ldp, n_plus, stride = 0, 0, 0
+    if plus is not None and plus.dim() == 3:
+        _need(plus.dtype == torch.float32 and plus.shape[1:] == (T, dim) and plus.stride(2) == 1,
+              "partial sums must be float32 [S, T, dim]")
+        ldp, n_plus, stride = plus.stride(1), plus.shape[0], plus.stride(0)
+    elif plus is not None:
         _need(plus.shape == (T, dim) and plus.stride(1) == 1, "plus must be [T, dim]")
+        ldp, n_plus = plus.stride(0), 1
     out = torch.empty((1, T, dim), dtype=torch.float32, device=y.device)
-    st = _lib.load("moe").fg_moe_combine(_ptr(y), _ptr(weight), _ptr(plus), plus.stride(0) if plus is not None else 0,
-                                         _code(plus) if plus is not None else F32, T, top, dim, _ptr(out), _stream(y))
+    st = _lib.load("moe").fg_moe_combine(_ptr(y), _ptr(weight), _ptr(plus), ldp, _code(plus) if plus is not None else F32,
+                                         n_plus, ctypes.c_longlong(stride), T, top, dim, _ptr(out), _stream(y))
     _check(st, "moe_combine")
     return out

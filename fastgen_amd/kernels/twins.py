@@ -375,7 +375,7 @@ def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tens
     T, top = weight.shape
     out = (weight[:, :, None] * y.view(T, top, -1)).sum(1)
     if plus is not None:
-        out = out + plus.float()
+        out = (plus.sum(0) if plus.dim() == 3 else plus.float()) + out
     return out[None]
 
 

@@ -75,7 +75,12 @@ class ParallelBlock:
             return mixed
         if getattr(self.ffn, "adds_to", False):
             return self.ffn.forward(x, plus=mixed)
-        return ops.add_rows(mixed, self.ffn.forward(x))
+        fed = self.ffn.forward(x)
+        if mixed.dim() == 3 or fed.dim() == 3:
+            # fp32 partial sums (products whose k range was cut): all of them are the norm's to add
+            as_parts = lambda t: t if t.dim() == 3 else t.float()[None]
+            return torch.cat([as_parts(mixed), as_parts(fed)])
+        return ops.add_rows(mixed, fed)
 
 
 register_part("arrangement", "parallel", lambda spec, *parts: ParallelBlock(*parts))

@@ -71,12 +71,20 @@ class MoE(FeedForward):
         self.w_down = place(down, MATRIX, dtype, device)
 
     def tile_rows(self, n_rows: int) -> int:
-        """Rows of one expert a tile holds: 16, or more where the experts get so many rows each that
-        their matrices would otherwise be read many times over (the matrix-core kernels only)."""
+        """Rows of one expert a tile holds: 16 for few rows (decode: an expert's matrices are read once for
+        its rows), more where the experts get so many rows each that their matrices would otherwise be
+        read many times over; from about a hundred rows an expert the tiles that go through LDS (the
+        matrix-core kernels only)."""
         if self.w_gate.dtype != torch.bfloat16 or self.dim % 8:
             return 16
         per_expert = n_rows * self.top / self.n_experts
-        return 64 if per_expert >= 48 else 32 if per_expert >= 24 else 16
+        lds_ok = min(self.dim, self.w_down.shape[2]) >= 32  # the tiles through LDS load k in steps of 32
+        # a tile is computed whole whatever it holds, and every expert's last tile is half empty on average:
+        # the largest tiles only where an expert has several of them
+        for rows, least in ((256, 768), (128, 96), (64, 48), (32, 24)):
+            if per_expert >= least and (rows < 128 or lds_ok):
+                return rows
+        return 16
 
     def forward(self, x: torch.Tensor, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
         """fp32 ``[1, T, dim]``: the experts' weighted sum (plus ``plus``, rows that go to the

@@ -90,11 +90,11 @@ def test_embedding_scale_offset_norm_and_stream_additions(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("D,E,top,F,T", [(64, 5, 2, 24, 70), (96, 4, 1, 20, 7), (40, 6, 6, 16, 33), (128, 3, 2, 64, 300),
-                                         (64, 70, 3, 8, 1)])
+                                         (64, 70, 3, 8, 1), (72, 4, 2, 44, 230), (64, 2, 1, 40, 90), (48, 3, 2, 20, 400)])
 def test_routed_experts_alone(dtype, D, E, top, F, T):
     """Router, sort, the experts' products and the weighted sum against the plain mixture: few rows (tiles of
-    16) and many rows an expert (larger tiles), all experts chosen, one chosen, more experts than a wave
-    has lanes, widths that are no multiple of 8."""
+    16) and many rows an expert (larger tiles, and those that go through LDS), all experts chosen, one
+    chosen, more experts than a wave has lanes, widths that are no multiple of 8 or of 32."""
     from fastgen_amd.config import PartSpec
     from fastgen_amd.kernels import ops
     from fastgen_amd.parts import build_part

@@ -463,7 +463,8 @@ def test_gemm_skinny_qkv_with_gate_and_values_from_the_keys_twin(ops, M, H, KV, 
 @gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,D,E,top,F,tile_rows", [(7, 72, 5, 2, 24, 16), (300, 136, 3, 2, 40, 64), (90, 64, 4, 4, 16, 32),
-                                                  (1, 40, 70, 3, 8, 16)])
+                                                  (1, 40, 70, 3, 8, 16), (300, 136, 3, 2, 40, 128), (700, 72, 2, 1, 56, 256),
+                                                  (260, 200, 5, 3, 328, 128)])
 def test_routed_expert_kernels_twins(ops, dtype, T, D, E, top, F, tile_rows):
     torch.manual_seed(T + E)
     if dtype == torch.float32:
@@ -482,16 +483,21 @@ def test_routed_expert_kernels_twins(ops, dtype, T, D, E, top, F, tile_rows):
     sorted_c, tiles_c = twins.moe_sort(choice, E, tile_rows)
     assert torch.equal(tiles_d.cpu(), tiles_c)
     # within an expert the kernel's order is free: the same pairs at each expert's places
-    for e, first, rows, _ in tiles_c.tolist():
-        assert sorted(sorted_d.cpu()[first:first + rows].tolist()) == sorted(sorted_c[first:first + rows].tolist())
+    first = 0
+    for c in torch.bincount(choice.reshape(-1).long(), minlength=E).tolist():
+        assert sorted(sorted_d.cpu()[first:first + c].tolist()) == sorted(sorted_c[first:first + c].tolist())
+        first += c
     wg, wu, wd = (torch.randn(E, F, D) / 4).to(dtype), (torch.randn(E, F, D) / 4).to(dtype), (torch.randn(E, D, F) / 4).to(dtype)
     act_d = ops.moe_gate_up(x.cuda(), wg.cuda(), wu.cuda(), sorted_d, tiles_d, top, tile_rows)
     act_c = twins.moe_gate_up(x, wg, wu, sorted_d.cpu(), tiles_c, top, tile_rows)
-    _close(act_d, act_c, dtype)
+    # (sums over a few hundred k in another order than the twin's: a few units of fp32 rounding more)
+    close = (lambda a, b: torch.testing.assert_close(a.cpu(), b, rtol=1e-4, atol=1e-4)) if dtype == torch.float32 else (
+        lambda a, b: _close(a, b, dtype))
+    close(act_d, act_c)
     y_d = ops.moe_down(act_d, wd.cuda(), sorted_d, tiles_d, tile_rows)
     y_c = twins.moe_down(act_d.cpu(), wd, sorted_d.cpu(), tiles_c, tile_rows)
-    _close(y_d, y_c, dtype)
+    close(y_d, y_c)
     plus = torch.randn(T, D).to(dtype)
-    for p in (None, plus):
+    for p in (None, plus, torch.randn(3, T, D)):
         got = ops.moe_combine(y_d, weight.cuda(), p.cuda() if p is not None else None)
         torch.testing.assert_close(got.cpu(), twins.moe_combine(y_d.cpu(), weight, p), rtol=1e-5, atol=1e-5)
