@@ -355,10 +355,16 @@ def _split_target_blocks() -> int:
 _SPLIT_MIN_TILES = int(os.environ.get("FG_SPLIT_MIN_TILES", 4))
 
 
-def attention_tile_rows(head_dim: int, small: bool = False) -> int:
+def _mfma_attention(head_dim: int, exact: bool = False):
+    """The matrix-core attention library for this head size: the plain build, or the one whose softmax
+    weights keep 16 significant bits (a model that asks for it loads only that one)."""
+    return _lib.load(f"attention_mfma_exact@{head_dim}" if exact else f"attention_mfma@{head_dim}")
+
+
+def attention_tile_rows(head_dim: int, small: bool = False, exact: bool = False) -> int:
     """Query rows of one item of the tile kernel for this head size: of its larger form (128 rows up to
     head size 128), or of the form with ``small`` items (64 rows, more and lighter workgroups)."""
-    return int(_lib.load(f"attention_mfma@{head_dim}").fg_attn_tile_rows(int(small)))
+    return int(_mfma_attention(head_dim, exact).fg_attn_tile_rows(int(small)))
 
 
 def attention_items(q_lens, q_start, n_cached, group_size: int, tile_rows: int = 64):
@@ -397,7 +403,7 @@ def _plan_ints(lib, max_chunks: int) -> int:
 
 
 def attention_plan(items: torch.Tensor, n_items: int, max_chunks: int, head_dim: int, window: int = 0,
-                   min_tiles: int = 4) -> torch.Tensor:
+                   min_tiles: int = 4, exact: bool = False) -> torch.Tensor:
     """Cuts the key ranges of ``items`` (device int32 ``[n_items, 4]``, 16-byte aligned) into chunks of
     the same number of 64-key tiles, a multiple of ``min_tiles``, on the device: a captured step cuts
     anew for the lengths of every replay.  The int32 plan that :func:`paged_attention_mfma` takes."""
@@ -405,7 +411,7 @@ def attention_plan(items: torch.Tensor, n_items: int, max_chunks: int, head_dim:
     _i32(items, "items")
     _need(items.data_ptr() % 16 == 0 and items.numel() >= 4 * n_items > 0, "items must be [n, 4], 16-byte aligned")
     _need(max_chunks >= 2 * n_items and min_tiles >= 1, "max_chunks must be at least twice the number of items")
-    lib = _lib.load(f"attention_mfma@{head_dim}")  # the plan is the same for every head size
+    lib = _mfma_attention(head_dim, exact)  # the plan is the same for every head size and build
     plan = torch.empty(_plan_ints(lib, max_chunks), dtype=torch.int32, device=items.device)
     _check(lib.fg_attn_plan(_ptr(items), n_items, int(window or 0), max_chunks, min_tiles, _ptr(plan),
                             _stream(items)), "attn_plan")
@@ -457,7 +463,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
     _need(out.shape == (T, n_heads * hd) and out.stride(1) == 1 and out.stride(0) % 4 == 0, "out must be [T, H*hd]")
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1,
           "block_table must be int32 [B, max_pages]")
-    lib = _lib.load(f"attention_mfma_exact@{hd}" if exact_weights else f"attention_mfma@{hd}")
+    lib = _mfma_attention(hd, exact_weights)
     G = n_heads // n_kv
     beside = None
     if (small_items is not None and small_items.numel() and big_items is not None and big_items.numel()
@@ -476,7 +482,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
             max_chunks = attention_chunks_for(n, n_kv)
         _need(2 * n <= max_chunks <= 65535, "the chunk list holds at least two chunks an item and at most 65535")
         if plan is None:
-            plan = attention_plan(small_items, n, max_chunks, hd, window, min_tiles)
+            plan = attention_plan(small_items, n, max_chunks, hd, window, min_tiles, exact_weights)
         _need(plan.dtype == torch.int32 and plan.numel() == _plan_ints(lib, max_chunks),
               "the plan does not fit the items and max_chunks")
         part_o = torch.empty((max_chunks * n_kv * 16, hd), dtype=torch.float32, device=q.device)
@@ -487,8 +493,9 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
             page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
         _check(st, "attn_split")
     if big_items is not None and big_items.numel():
-        tile_rows = attention_tile_rows(hd) if tile_rows is None else int(tile_rows)
-        _need(tile_rows in (attention_tile_rows(hd), attention_tile_rows(hd, True)), "tile_rows is no form of the tile kernel")
+        tile_rows = attention_tile_rows(hd, False, exact_weights) if tile_rows is None else int(tile_rows)
+        _need(tile_rows in (attention_tile_rows(hd, False, exact_weights), attention_tile_rows(hd, True, exact_weights)),
+              "tile_rows is no form of the tile kernel")
         _need(G <= tile_rows, "too many query heads per kv head for the tile kernel")
         _i32(big_items, "big_items")
         _need(big_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
@@ -527,13 +534,13 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
             # already (and are refreshed with it when the step is a replayed graph)
             plan = (ctx.seq_records, None, ctx.n_seqs, None)
         else:
-            tile_rows = attention_tile_rows(hd)
+            tile_rows = attention_tile_rows(hd, False, exact_weights)
             small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G, tile_rows)
-            if 0 < len(big) * n_kv <= compute_units() // 2 and attention_tile_rows(hd, True) < tile_rows:
+            if 0 < len(big) * n_kv <= compute_units() // 2 and attention_tile_rows(hd, True, exact_weights) < tile_rows:
                 # so few items that half the compute units would stand idle: items of half the rows, whose
                 # lighter workgroups share a unit (prompt portions of up to 512 tokens: 11.6 / 17.6 us
                 # against 14.1 / 19.5 at 256 / 512 tokens; equal at 1,024, slower beyond)
-                tile_rows = attention_tile_rows(hd, True)
+                tile_rows = attention_tile_rows(hd, True, exact_weights)
                 small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G, tile_rows)
             both = upload(np.concatenate([small, big]).reshape(-1), torch.int32, q.device)
             plan = (both[: small.size] if small.size else None, both[small.size:] if big.size else None, len(small),
@@ -547,7 +554,8 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
         key = ("attention_plan", G, int(window or 0), chunks)
         split_plan = ctx.scratch.get(key)
         if split_plan is None:
-            split_plan = ctx.scratch[key] = attention_plan(small_d, n_small, chunks, hd, window, _SPLIT_MIN_TILES)
+            split_plan = ctx.scratch[key] = attention_plan(small_d, n_small, chunks, hd, window, _SPLIT_MIN_TILES,
+                                                           exact_weights)
     # rows of the largest small item: one token a sequence in a decode step (also a captured one)
     rows = G * int(ctx.q_lens.max()) if big_d is None else 16
     return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
