@@ -193,7 +193,7 @@ BUDERAX_SIZES = {
 
 def _buderax_configs(z: dict):
     mixer = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5,
-                 rot=dict(base=500000.0, dims=z["dim"], scaling=dict(factor=4.0)))
+                 rot=dict(base=1000000.0, dims=z["dim"] // 2, scaling=dict(factor=8.0)))
     mlp = dict(kind="moe", router=dict(experts=z["experts"], top=z["top"]), expert=dict(ff=z["ff"]))
     new = dict(architecture="Buderax", width=z["width"], vocab=z["vocab"], embedding=dict(scale=2.0), norm=dict(eps=1e-6),
                layers=[dict(type="attention", mixer=mixer, mlp=mlp) for _ in range(z["layers"])])
