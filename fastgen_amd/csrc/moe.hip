@@ -1,7 +1,7 @@
 // A routed feed-forward (mixture of experts) on the device, without a look of the host at what went
 // where, so that a step with it can be recorded:
 //
-//  route    per token: fp32 router logits (x W_r^T + b), the `top` largest, softmax over those
+//  route    per token (a workgroup): fp32 router logits (x W_r^T + b), the `top` largest, softmax over those
 //  sort     the (token, choice) pairs ordered by expert, cut into tiles of at most TM rows of one expert
 //  gate_up  per tile: act = silu(x W_gate^T) * (x W_up^T) with the expert's matrices, rows gathered by token
 //  down     per tile: y[pair] = act W_down^T in fp32, one row per pair
@@ -20,60 +20,51 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ------------------------------------------------------------------- route
-// Logits: a wave computes ROUTE_EPW experts' logits of one token (the row of x is read once for them),
-// eight elements a lane and round; lanes' partial sums are added by the wave in a fixed order.
-#define ROUTE_EPW 4
-template <class T>
-__global__ __launch_bounds__(256) void moe_logits_kernel(
+// A workgroup a token.  Logits: the WAVES waves take the experts in turns of EPW (a wave reads the row of
+// x once for its EPW experts, eight elements a lane and round; the lanes' partial sums are added by the
+// wave in a fixed order), into LDS.  Few tokens (decode) get 16 waves a token and 2 experts a turn, so that
+// the router's rows are asked for by many waves at once; many tokens 4 waves and 4 experts a turn.  Then the `top` largest (ties: the lower expert) by a
+// wave-wide argmax repeated `top` times, and the softmax over them; every wave does this on the same LDS
+// values, the first one stores.  LDS: n_experts logits, then `top` chosen values.
+template <class T, int WAVES, int EPW>
+__global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
     const T* __restrict__ x, int ldx, const float* __restrict__ wr, const float* __restrict__ bias,
-    int n_tokens, int dim, int n_experts, float* __restrict__ z) {
+    int dim, int n_experts, int top, int* __restrict__ choice, float* __restrict__ weight) {
+  extern __shared__ float lds[];
+  float* z = lds;
+  float* chosen = lds + n_experts;
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
-  const int groups = (n_experts + ROUTE_EPW - 1) / ROUTE_EPW;
-  const long long item = (long long)blockIdx.x * 4 + wave;
-  if (item >= (long long)n_tokens * groups) return;
-  const int t = (int)(item / groups), e0 = (int)(item % groups) * ROUTE_EPW;
-  const T* xr = x + (size_t)t * ldx;
-  float s[ROUTE_EPW];
+  const size_t t = blockIdx.x;
+  const T* xr = x + t * ldx;
+  for (int e0 = wave * EPW; e0 < n_experts; e0 += WAVES * EPW) {
+    float s[EPW];
 #pragma unroll
-  for (int j = 0; j < ROUTE_EPW; ++j) s[j] = 0.f;
-  if (dim % 8 == 0 && ldx % 8 == 0) {
-    for (int k = lane * 8; k < dim; k += FG_WAVE * 8) {
-      float xv[8];
-      load8<T>(xr + k, xv);
+    for (int j = 0; j < EPW; ++j) s[j] = 0.f;
+    if (dim % 8 == 0 && ldx % 8 == 0) {
+      for (int k = lane * 8; k < dim; k += FG_WAVE * 8) {
+        float xv[8];
+        load8<T>(xr + k, xv);
 #pragma unroll
-      for (int j = 0; j < ROUTE_EPW; ++j) {
-        float wv[8];
-        load8<float>(wr + (size_t)min(e0 + j, n_experts - 1) * dim + k, wv);
+        for (int j = 0; j < EPW; ++j) {
+          float wv[8];
+          load8<float>(wr + (size_t)min(e0 + j, n_experts - 1) * dim + k, wv);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) s[j] = fmaf(xv[i], wv[i], s[j]);
+          for (int i = 0; i < 8; ++i) s[j] = fmaf(xv[i], wv[i], s[j]);
+        }
+      }
+    } else {
+      for (int k = lane; k < dim; k += FG_WAVE) {
+        const float xv = to_f<T>(xr[k]);
+#pragma unroll
+        for (int j = 0; j < EPW; ++j) s[j] = fmaf(xv, wr[(size_t)min(e0 + j, n_experts - 1) * dim + k], s[j]);
       }
     }
-  } else {
-    for (int k = lane; k < dim; k += FG_WAVE) {
-      const float xv = to_f<T>(xr[k]);
 #pragma unroll
-      for (int j = 0; j < ROUTE_EPW; ++j) s[j] = fmaf(xv, wr[(size_t)min(e0 + j, n_experts - 1) * dim + k], s[j]);
+    for (int j = 0; j < EPW; ++j) {
+      const float v = wave_sum(s[j]);
+      if (lane == 0 && e0 + j < n_experts) z[e0 + j] = v + (bias ? bias[e0 + j] : 0.f);
     }
   }
-#pragma unroll
-  for (int j = 0; j < ROUTE_EPW; ++j) {
-    const float v = wave_sum(s[j]);
-    if (lane == 0 && e0 + j < n_experts) z[(size_t)t * n_experts + e0 + j] = v + (bias ? bias[e0 + j] : 0.f);
-  }
-}
-
-// The `top` largest logits of a token (ties: the lower expert) and the softmax over them: a wave a token.
-// LDS per wave: n_experts logits, then `top` chosen values.
-__global__ __launch_bounds__(256) void moe_topk_kernel(
-    const float* __restrict__ zg, int n_tokens, int n_experts, int top, int* __restrict__ choice,
-    float* __restrict__ weight) {
-  extern __shared__ float lds[];
-  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
-  const int t_raw = blockIdx.x * 4 + wave;
-  const int t = min(t_raw, n_tokens - 1);  // a wave beyond the tokens does the last one again and stores nothing
-  float* z = lds + (size_t)wave * (n_experts + top);
-  float* chosen = z + n_experts;
-  for (int e = lane; e < n_experts; e += FG_WAVE) z[e] = zg[(size_t)t * n_experts + e];
   __syncthreads();
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
@@ -88,40 +79,41 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(
       const int oa = __shfl_xor(at, m, FG_WAVE);
       if (ov > best || (ov == best && oa < at)) { best = ov; at = oa; }
     }
-    __syncthreads();
-    if (lane == 0) {
+    __syncthreads();  // every wave has read the logits of this turn
+    if (threadIdx.x == 0) {
       at = min(at, n_experts - 1);  // (only if every logit is NaN)
       z[at] = -INFINITY;
       chosen[j] = best;
-      if (t_raw < n_tokens) choice[(size_t)t * top + j] = at;
+      choice[t * top + j] = at;
     }
     __syncthreads();
   }
-  if (lane == 0 && t_raw < n_tokens) {
+  if (threadIdx.x == 0) {
     const float m = chosen[0];  // the largest
     float sum = 0.f;
     for (int j = 0; j < top; ++j) sum += expf(chosen[j] - m);
-    for (int j = 0; j < top; ++j) weight[(size_t)t * top + j] = expf(chosen[j] - m) / sum;
+    for (int j = 0; j < top; ++j) weight[t * top + j] = expf(chosen[j] - m) / sum;
   }
 }
 
-// z: fp32 scratch [n_tokens, n_experts] for the logits
 extern "C" int fg_moe_route(const void* x, int ldx, int dtype, const float* wr, const float* bias, int n_tokens, int dim,
-                            int n_experts, int top, float* z, int* choice, float* weight, hipStream_t stream) {
+                            int n_experts, int top, int* choice, float* weight, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
-  if (dim <= 0 || ldx < dim || n_experts <= 0 || top < 1 || top > n_experts || !z) return FG_ERR_ARG;
-  const size_t lds = (size_t)4 * (n_experts + top) * sizeof(float);
+  if (dim <= 0 || ldx < dim || n_experts <= 0 || top < 1 || top > n_experts) return FG_ERR_ARG;
+  const size_t lds = (size_t)(n_experts + top) * sizeof(float);
   if (lds > 60000) return FG_ERR_ARG;
-  const long long items = (long long)n_tokens * ((n_experts + ROUTE_EPW - 1) / ROUTE_EPW);
-  if ((items + 3) / 4 > 2147483647LL) return FG_ERR_ARG;
-  const unsigned blocks = (unsigned)((items + 3) / 4);
-  if (dtype == FG_F32)
-    moe_logits_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, ldx, wr, bias, n_tokens, dim, n_experts, z);
-  else if (dtype == FG_BF16)
-    moe_logits_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, wr, bias, n_tokens, dim, n_experts, z);
-  else
+#define GO(T, WAVES, EPW)                                                                                        \
+  moe_route_kernel<T, WAVES, EPW><<<n_tokens, 64 * WAVES, lds, stream>>>((const T*)x, ldx, wr, bias, dim, n_experts, \
+                                                                         top, choice, weight)
+  const bool few = n_tokens <= 64;
+  if (dtype == FG_F32) {
+    if (few) GO(float, 16, 2); else GO(float, 4, 4);
+  } else if (dtype == FG_BF16) {
+    if (few) GO(bf16_t, 16, 2); else GO(bf16_t, 4, 4);
+  } else {
     return FG_ERR_ARG;
-  moe_topk_kernel<<<(n_tokens + 3) / 4, 256, lds, stream>>>(z, n_tokens, n_experts, top, choice, weight);
+  }
+#undef GO
   return fg_launch_status();
 }
 
@@ -270,22 +262,27 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
   f32x4 ag[MB], au[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) ag[mb] = au[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 8 * g; k0 < dim + 8 * g; k0 += 64) {  // this lane's k: 8 g, 8 g + 32, ...
-    bf16x8 a0 = load_k(pg, k0, dim), a1 = load_k(pg, k0 + 32, dim);
-    bf16x8 u0 = load_k(pu, k0, dim), u1 = load_k(pu, k0 + 32, dim);
-    bf16x8 b0[MB], b1[MB];
+  // U steps of 32 k a round, all their loads issued before the first MFMA: with few rows a wave is a chain of
+  // memory round trips, and the fewer of them the better (8 steps for one block of rows: 24 loads in flight)
+  constexpr int U = MB == 1 ? 8 : (MB == 2 ? 4 : 2);
+  for (int k0 = 8 * g; k0 < dim + 8 * g; k0 += 32 * U) {  // this lane's k: 8 g, 8 g + 32, ...
+    bf16x8 a[U], u[U], b[U][MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      b0[mb] = load_k(px[mb], k0, dim);
-      b1[mb] = load_k(px[mb], k0 + 32, dim);
+    for (int i = 0; i < U; ++i) {
+      a[i] = load_k(pg, k0 + 32 * i, dim);
+      u[i] = load_k(pu, k0 + 32 * i, dim);
     }
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      ag[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0[mb], ag[mb], 0, 0, 0);
-      au[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u0, b0[mb], au[mb], 0, 0, 0);
-      ag[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1[mb], ag[mb], 0, 0, 0);
-      au[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u1, b1[mb], au[mb], 0, 0, 0);
-    }
+    for (int i = 0; i < U; ++i)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) b[i][mb] = load_k(px[mb], k0 + 32 * i, dim);
+#pragma unroll
+    for (int i = 0; i < U; ++i)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        ag[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[i][mb], ag[mb], 0, 0, 0);
+        au[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[i], b[i][mb], au[mb], 0, 0, 0);
+      }
   }
   // the lane holds, for the tile's row mb * 16 + r16, channels c0 + 4 g .. + 3
 #pragma unroll
@@ -326,19 +323,19 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
   f32x4 acc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 8 * g; k0 < hidden + 8 * g; k0 += 64) {
-    bf16x8 a0 = load_k(pw, k0, hidden), a1 = load_k(pw, k0 + 32, hidden);
-    bf16x8 b0[MB], b1[MB];
+  constexpr int U = MB == 1 ? 8 : (MB == 2 ? 4 : 2);  // as in gate_up
+  for (int k0 = 8 * g; k0 < hidden + 8 * g; k0 += 32 * U) {
+    bf16x8 a[U], b[U][MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      b0[mb] = load_k(pa[mb], k0, hidden);
-      b1[mb] = load_k(pa[mb], k0 + 32, hidden);
-    }
+    for (int i = 0; i < U; ++i) a[i] = load_k(pw, k0 + 32 * i, hidden);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0[mb], acc[mb], 0, 0, 0);
-      acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1[mb], acc[mb], 0, 0, 0);
-    }
+    for (int i = 0; i < U; ++i)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) b[i][mb] = load_k(pa[mb], k0 + 32 * i, hidden);
+#pragma unroll
+    for (int i = 0; i < U; ++i)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[i][mb], acc[mb], 0, 0, 0);
   }
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {

@@ -917,9 +917,8 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     _need(1 <= top <= E, f"top={top} must be between 1 and the {E} experts")
     choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weight = torch.empty((T, top), dtype=torch.float32, device=x.device)
-    logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
     st = _lib.load("moe").fg_moe_route(_ptr(x), x.stride(0), _code(x), _ptr(router), _ptr(bias), T, dim, E, top,
-                                       _ptr(logits), _ptr(choice), _ptr(weight), _stream(x))
+                                       _ptr(choice), _ptr(weight), _stream(x))
     _check(st, "moe_route")
     return choice, weight
 
