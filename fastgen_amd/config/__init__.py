@@ -9,6 +9,7 @@ from .registry import (
 )
 from . import llama as _llama  # registers LlamaForCausalLM
 from . import buderax as _buderax  # registers Buderax
+from . import gisodra as _gisodra  # registers Gisodra
 
 __all__ = [
     "Architecture",

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(ATT_WAVES* FG_WAVE) void paged_attention_general_ke
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, int n_tokens, int n_heads, int n_kv, int hd,
-    int page_size, float scale, int window) {
+    int page_size, float scale, int window, const float* __restrict__ sinks) {
   __shared__ float q_s[ATT_WAVES][ATT_MAX_HD];
   __shared__ float p_s[ATT_WAVES][ATT_TILE];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
@@ -133,6 +133,8 @@ __global__ __launch_bounds__(ATT_WAVES* FG_WAVE) void paged_attention_general_ke
     __builtin_amdgcn_wave_barrier();
   }
   T* orow = out + (size_t)t * out_stride + (size_t)h * hd;
+  // a sink: one more term exp(sinks[h]) in the softmax's denominator, which brings no value
+  if (sinks) l += expf(sinks[h] - m);
   const float inv = 1.f / l;
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) {
@@ -141,11 +143,11 @@ __global__ __launch_bounds__(ATT_WAVES* FG_WAVE) void paged_attention_general_ke
   }
 }
 
-extern "C" int fg_paged_attention_general(
+extern "C" int fg_paged_attention_general_sink(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
     const void* v_pages, const int* block_table, int bt_stride, const int* seq_of_token,
     const int* positions, int n_tokens, int n_heads, int n_kv, int hd, int page_size,
-    float scale, int window, int dtype, hipStream_t stream) {
+    float scale, int window, const float* sinks, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
   if (hd <= 0 || hd % 8 || hd > ATT_MAX_HD || page_size <= 0 || page_size % 8 || n_kv <= 0 ||
       n_heads <= 0 || n_heads % n_kv || window < 0)
@@ -158,13 +160,23 @@ extern "C" int fg_paged_attention_general(
     paged_attention_general_kernel<float><<<grid, ATT_WAVES * FG_WAVE, 0, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_pages,
         (const float*)v_pages, block_table, bt_stride, seq_of_token, positions, n_tokens,
-        n_heads, n_kv, hd, page_size, scale, window);
+        n_heads, n_kv, hd, page_size, scale, window, sinks);
   else if (dtype == FG_BF16)
     paged_attention_general_kernel<bf16_t><<<grid, ATT_WAVES * FG_WAVE, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
         (const bf16_t*)v_pages, block_table, bt_stride, seq_of_token, positions, n_tokens,
-        n_heads, n_kv, hd, page_size, scale, window);
+        n_heads, n_kv, hd, page_size, scale, window, sinks);
   else
     return FG_ERR_ARG;
   return fg_launch_status();
+}
+
+extern "C" int fg_paged_attention_general(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+    const void* v_pages, const int* block_table, int bt_stride, const int* seq_of_token,
+    const int* positions, int n_tokens, int n_heads, int n_kv, int hd, int page_size,
+    float scale, int window, int dtype, hipStream_t stream) {
+  return fg_paged_attention_general_sink(q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_stride,
+                                         seq_of_token, positions, n_tokens, n_heads, n_kv, hd, page_size, scale,
+                                         window, nullptr, dtype, stream);
 }

@@ -354,7 +354,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ plan,
     float* __restrict__ part_o, float* __restrict__ part_ml, int n_heads, int n_kv, int page_size,
-    int page_shift, float scale, int window) {
+    int page_shift, float scale, int window, const float* __restrict__ sinks) {
   __shared__ float o_s[2][16][HD + 1];
   __shared__ float ml_s[2][16][2];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
@@ -482,6 +482,8 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   const int t_out = it.tok0 + r16 / G, h_out = kvh * G + r16 % G;
   if (alone) {
     bf16_t* orow = out + (size_t)t_out * out_stride + (size_t)h_out * HD;
+    // a sink: one more term exp(sink) in the denominator (maxima are in base 2 and scaled), no value
+    if (sinks) l += __builtin_amdgcn_exp2f(sinks[h_out] * LOG2E - m);
     const float inv = 1.f / l;
 #pragma unroll
     for (int db = 0; db < NDB; ++db) {
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
 // wave, one chunk a lane, together with the first eight partial outputs.
 __global__ void attn_combine_rows_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                     const int* __restrict__ plan, bf16_t* __restrict__ out, int out_stride,
-                                    int n_heads, int n_kv) {
+                                    int n_heads, int n_kv, const float* __restrict__ sinks) {
   __shared__ float f_s[COMBINE_MAX_SPLITS];  // weight of each chunk's partial output: 2^(m_s - M) / L
   const int r = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z, d = threadIdx.x;
   const int G = n_heads / n_kv;
@@ -548,6 +550,7 @@ __global__ void attn_combine_rows_kernel(const float* __restrict__ part_o, const
       L += ms[j] * ls[j];
     }
     L = wave_sum(L);
+    if (sinks) L += __builtin_amdgcn_exp2f(sinks[kvh * G + r % G] * LOG2E - M);
     const float inv = 1.f / L;
 #pragma unroll
     for (int j = 0; j < PER; ++j) f_s[threadIdx.x + j * FG_WAVE] = ms[j] * inv;
@@ -573,7 +576,7 @@ __global__ void attn_combine_rows_kernel(const float* __restrict__ part_o, const
 // lane; then every thread adds up four neighbouring head dimensions of a row (or of several rows).
 __global__ __launch_bounds__(256) void attn_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ plan,
-    bf16_t* __restrict__ out, int out_stride, int n_heads, int n_kv) {
+    bf16_t* __restrict__ out, int out_stride, int n_heads, int n_kv, const float* __restrict__ sinks) {
   __shared__ float f_s[16][COMBINE_MAX_SPLITS];  // weight of each chunk's partial output: 2^(m_s - M) / L
   const int kvh = blockIdx.x, chunk = blockIdx.y, tid = threadIdx.x;
   const int lane = tid % FG_WAVE, wave = tid / FG_WAVE;
@@ -616,6 +619,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(
       L += ms[j] * ls[j];
     }
     L = wave_sum(L);
+    if (sinks) L += __builtin_amdgcn_exp2f(sinks[kvh * G + (4 * wave + rr) % G] * LOG2E - M);
     const float inv = 1.f / L;  // (a row beyond the item's: never stored)
 #pragma unroll
     for (int j = 0; j < PER; ++j) f_s[4 * wave + rr][lane + j * FG_WAVE] = ms[j] * inv;
@@ -670,11 +674,13 @@ extern "C" int fg_attn_plan(const int* items, int n_items, int window, int max_c
 // plan: what fg_attn_plan made of the items, with the same n_items, max_chunks and window.
 // max_rows: no item has more rows (tokens x heads of a kv head's group) than this, at most 16.
 // part_o: fp32 [max_chunks * n_kv * 16 * HD], part_ml: the same rows x 2.
-extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
-                             const void* v_pages, const int* block_table, int bt_stride, const int* plan,
-                             int n_items, int max_chunks, int max_rows, float* part_o, float* part_ml,
-                             int n_heads, int n_kv, int hd, int page_size, float scale, int window,
-                             hipStream_t stream) {
+// sinks: fp32 [n_heads] or null: head h's softmax has one more term exp(sinks[h]) in its denominator, which
+// brings no value.
+extern "C" int fg_attn_split_sink(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                                  const void* v_pages, const int* block_table, int bt_stride, const int* plan,
+                                  int n_items, int max_chunks, int max_rows, float* part_o, float* part_ml,
+                                  int n_heads, int n_kv, int hd, int page_size, float scale, int window,
+                                  const float* sinks, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || page_size < 8 || page_size % 8 ||
       !(scale > 0.f) || max_chunks < 2 * n_items || max_chunks > 65535 || n_kv > 65535 || window < 0 ||
@@ -684,16 +690,26 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
   attn_split_kernel<PERM><<<dim3(n_kv, max_chunks), 256, 0, stream>>>(                                         \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,    \
       block_table, bt_stride, plan, part_o, part_ml, n_heads, n_kv, page_size,                                 \
-      page_shift_of(page_size), scale, window)
+      page_shift_of(page_size), scale, window, sinks)
   if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
 #undef LAUNCH
   if ((long long)max_chunks * n_kv * max_rows <= COMBINE_ROWS_MAX_GROUPS)
     attn_combine_rows_kernel<<<dim3(max_rows, n_kv, max_chunks), HD < 64 ? 64 : HD, 0, stream>>>(
-        part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv);
+        part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv, sinks);
   else
     attn_combine_kernel<<<dim3(n_kv, max_chunks), 256, 0, stream>>>(
-        part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv);
+        part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv, sinks);
   return fg_launch_status();
+}
+
+extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                             const void* v_pages, const int* block_table, int bt_stride, const int* plan,
+                             int n_items, int max_chunks, int max_rows, float* part_o, float* part_ml,
+                             int n_heads, int n_kv, int hd, int page_size, float scale, int window,
+                             hipStream_t stream) {
+  return fg_attn_split_sink(q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_stride, plan, n_items,
+                            max_chunks, max_rows, part_o, part_ml, n_heads, n_kv, hd, page_size, scale, window,
+                            nullptr, stream);
 }
 
 // ----------------------------------------------------------- without allocation
@@ -801,7 +817,7 @@ __global__ __launch_bounds__(TILE_PAIR ? 512 : 256, TILE_PAIR ? 1 : 2) void attn
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_heads, int n_kv,
-    int page_size, int page_shift, float scale, int window) {
+    int page_size, int page_shift, float scale, int window, const float* __restrict__ sinks) {
   constexpr int TILE_RB = TILE_PAIR ? 2 : 1;  // row blocks a wave holds
   constexpr int TILE_THREADS = TILE_PAIR ? 512 : 256;
   constexpr int NT = TILE_THREADS;
@@ -1060,6 +1076,7 @@ __global__ __launch_bounds__(TILE_PAIR ? 512 : 256, TILE_PAIR ? 1 : 2) void attn
     const int row = (rg * RB + rb) * 16 + r16;
     if (row < it.n_tok * G) {
       bf16_t* orow = out + (size_t)(it.tok0 + row / G) * out_stride + (size_t)(kvh * G + row % G) * HD;
+      if (sinks) lsum += __builtin_amdgcn_exp2f(sinks[kvh * G + row % G] * LOG2E - m[rb]);
       const float inv = 1.f / lsum;
 #pragma unroll
       for (int db = 0; db < NDB; ++db) {
@@ -1075,13 +1092,13 @@ __global__ __launch_bounds__(TILE_PAIR ? 512 : 256, TILE_PAIR ? 1 : 2) void attn
 struct TileArgs {
   const bf16_t* q; int q_stride; bf16_t* out; int out_stride; const bf16_t* k_pages; const bf16_t* v_pages;
   const int* block_table; int bt_stride; const int* items; int n_items, n_heads, n_kv, page_size; float scale;
-  int window; hipStream_t stream;
+  int window; const float* sinks; hipStream_t stream;
 };
 template <bool PERM, bool PAIR>
 static void launch_tile(const TileArgs& a) {
   attn_tile_kernel<PERM, PAIR><<<a.n_items * a.n_kv, PAIR ? 512 : 256, 0, a.stream>>>(
       a.q, a.q_stride, a.out, a.out_stride, a.k_pages, a.v_pages, a.block_table, a.bt_stride, a.items, a.n_heads,
-      a.n_kv, a.page_size, page_shift_of(a.page_size), a.scale, a.window);
+      a.n_kv, a.page_size, page_shift_of(a.page_size), a.scale, a.window, a.sinks);
 }
 // the form with two tiles at a time exists up to head size 128 only (its LDS)
 template <bool EXISTS> struct PairForm {
@@ -1092,21 +1109,29 @@ template <bool EXISTS> struct PairForm {
 template <> struct PairForm<false> { static void go(const TileArgs&) {} };
 
 // item_rows: the rows an item has at most, fg_attn_tile_rows(0) or fg_attn_tile_rows(1): which form of the kernel runs.
-extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
-                            const void* v_pages, const int* block_table, int bt_stride, const int* items,
-                            int n_items, int item_rows, int n_heads, int n_kv, int hd, int page_size, float scale,
-                            int window, hipStream_t stream) {
+extern "C" int fg_attn_tile_sink(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                                 const void* v_pages, const int* block_table, int bt_stride, const int* items,
+                                 int n_items, int item_rows, int n_heads, int n_kv, int hd, int page_size,
+                                 float scale, int window, const float* sinks, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || !(scale > 0.f) || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > item_rows || page_size < 8 || page_size % 8 ||
       (long long)n_items * n_kv > 2147483647LL || window < 0 || q_stride % 8 || out_stride % 4 ||
       (item_rows != TILE_ROWS && item_rows != TILE_ROWS_SMALL))
     return FG_ERR_ARG;
   const TileArgs a{(const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-                   block_table, bt_stride, items, n_items, n_heads, n_kv, page_size, scale, window, stream};
+                   block_table, bt_stride, items, n_items, n_heads, n_kv, page_size, scale, window, sinks, stream};
   if (TILE_PAIR_OK && item_rows == TILE_ROWS) PairForm<TILE_PAIR_OK>::go(a);
   else if (page_size % 32 == 0) launch_tile<true, false>(a);
   else launch_tile<false, false>(a);
   return fg_launch_status();
+}
+
+extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                            const void* v_pages, const int* block_table, int bt_stride, const int* items,
+                            int n_items, int item_rows, int n_heads, int n_kv, int hd, int page_size, float scale,
+                            int window, hipStream_t stream) {
+  return fg_attn_tile_sink(q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_stride, items, n_items,
+                           item_rows, n_heads, n_kv, hd, page_size, scale, window, nullptr, stream);
 }
 
 // query rows (tokens x heads of a kv head's group) of one item of fg_attn_tile: of the larger form, or

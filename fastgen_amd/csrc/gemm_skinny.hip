@@ -52,6 +52,16 @@ __device__ __forceinline__ WSrc w_src(const bf16_t* w, int ldw, int n0, int N, i
 #define EPI_SILU_MUL 1
 #define EPI_ROPE_KV 2  // w = [q; k; v] projections: rotate q and k, q to y, k and v into their cache pages
 #define EPI_RESIDUAL 3  // the product is added to the fp32 residual stream; see Residual
+#define EPI_GELU_MUL 4  // as EPI_SILU_MUL with another activation
+
+// silu(gate) * up, or with EPI_GELU_MUL the tanh form of GELU: 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * up
+#define EPI_IS_GATED(e) ((e) == EPI_SILU_MUL || (e) == EPI_GELU_MUL)
+template <int EPI>
+__device__ __forceinline__ float fg_gated(float gate, float up) {
+  if (EPI == EPI_GELU_MUL)
+    return 0.5f * gate * (1.f + tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate))) * up;
+  return gate / (1.f + __expf(-gate)) * up;
+}
 
 // For at most 16 rows the two RMSNorms of a layer need no kernels of their own.  The product that
 // feeds the residual stream (EPI_RESIDUAL) adds its result to h, stores h * norm_w (not yet divided by
@@ -233,7 +243,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
         up *= rscale[m];
       }
       const int col = n0 / 2 + j;
-      if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + col] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
+      if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + col] = from_f<TY>(fg_gated<EPI>(gate, up));
     }
   }
 }
@@ -378,7 +388,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
       }
       gate *= rscale[m];
       up *= rscale[m];
-      if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + n0 / 2 + j] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
+      if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + n0 / 2 + j] = from_f<TY>(fg_gated<EPI>(gate, up));
     }
   }
 }
@@ -475,7 +485,7 @@ __global__ __launch_bounds__(256, MB <= 4 ? 3 : 2) void gemm_skinny64_kernel(
         const float other = __shfl_xor(acc[mb][i], 32, FG_WAVE);
         const float gate = acc[mb][i], up = other;
         const int col = n0 / 2 + 4 * g + i;
-        if (g < 2 && m < M && n0 + 8 + 4 * g + i < N) yp[(size_t)m * ldy + col] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
+        if (g < 2 && m < M && n0 + 8 + 4 * g + i < N) yp[(size_t)m * ldy + col] = from_f<TY>(fg_gated<EPI>(gate, up));
       }
     }
   }
@@ -511,9 +521,9 @@ extern "C" int fg_gemm_skinny(const void* x, int ldx, const void* w, int ldw, vo
                               int K, int out_dtype, int epilogue, hipStream_t stream) {
   if (M <= 0 || N <= 0) return FG_OK;
   if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K)) return FG_ERR_ARG;
-  if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2)) return FG_ERR_ARG;
+  if (EPI_IS_GATED(epilogue) && (N % 16 || ldy < N / 2)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && ldy < N) return FG_ERR_ARG;
-  if (epilogue != EPI_STORE && epilogue != EPI_SILU_MUL) return FG_ERR_ARG;
+  if (epilogue != EPI_STORE && !EPI_IS_GATED(epilogue)) return FG_ERR_ARG;
   const int mb = (M + 15) / 16;
   const RowScale sc{nullptr, 0, 0.f, 0.f};
   const Residual rs{};
@@ -525,6 +535,8 @@ extern "C" int fg_gemm_skinny(const void* x, int ldx, const void* w, int ldw, vo
       launch_skinny<MB, EPI_STORE, float>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);           \
     else if (epilogue == EPI_SILU_MUL && out_dtype == FG_BF16)                                        \
       launch_skinny<MB, EPI_SILU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);       \
+    else if (epilogue == EPI_GELU_MUL && out_dtype == FG_BF16)                                        \
+      launch_skinny<MB, EPI_GELU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);       \
     else                                                                                              \
       return FG_ERR_ARG;                                                                              \
   } while (0)
@@ -548,7 +560,7 @@ extern "C" int fg_gemm_skinny_fused(const void* x, int ldx, const void* w, int l
   if (M <= 0 || N <= 0) return FG_OK;
   if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K)) return FG_ERR_ARG;
   if (ssq && (n_parts < 1 || dim < 1 || !(eps >= 0.f))) return FG_ERR_ARG;
-  if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || !y)) return FG_ERR_ARG;
+  if (EPI_IS_GATED(epilogue) && (N % 16 || ldy < N / 2 || !y)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && (ldy < N || !y)) return FG_ERR_ARG;
   if (epilogue == EPI_RESIDUAL && (!h || !norm_w || !x_out || !ssq_out || ldh < N || ldxo < N ||
                                    (norm_w_dtype != FG_F32 && norm_w_dtype != FG_BF16)))
@@ -557,6 +569,7 @@ extern "C" int fg_gemm_skinny_fused(const void* x, int ldx, const void* w, int l
   const Residual rs{h, ldh, norm_w, norm_w_dtype == FG_F32, (bf16_t*)x_out, ldxo, ssq_out};
   if (epilogue == EPI_STORE) launch_skinny<1, EPI_STORE, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);
   else if (epilogue == EPI_SILU_MUL) launch_skinny<1, EPI_SILU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);
+  else if (epilogue == EPI_GELU_MUL) launch_skinny<1, EPI_GELU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);
   else if (epilogue == EPI_RESIDUAL) launch_skinny<1, EPI_RESIDUAL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);
   else return FG_ERR_ARG;
   return fg_launch_status();
@@ -576,9 +589,9 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
   const RowScale sc{ssq, n_parts, ssq ? 1.f / (float)dim : 0.f, eps};
   if (M > 128 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K) || k_splits < 1 || k_splits > 65535)
     return FG_ERR_ARG;
-  if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
+  if (EPI_IS_GATED(epilogue) && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && (ldy < N || (k_splits > 1 && out_dtype != FG_F32))) return FG_ERR_ARG;
-  if (epilogue != EPI_STORE && epilogue != EPI_SILU_MUL) return FG_ERR_ARG;
+  if (epilogue != EPI_STORE && !EPI_IS_GATED(epilogue)) return FG_ERR_ARG;
   const int k_per_split = ((K + k_splits * 256 - 1) / (k_splits * 256)) * 256;
   const dim3 grid((N + 63) / 64, k_splits);
   const int mb = (M + 15) / 16;
@@ -588,6 +601,7 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
 #define PICK(MB)                                                                   \
   do {                                                                             \
     if (epilogue == EPI_SILU_MUL) GO64(MB, EPI_SILU_MUL, bf16_t);                  \
+    else if (epilogue == EPI_GELU_MUL) GO64(MB, EPI_GELU_MUL, bf16_t);             \
     else if (out_dtype == FG_BF16) GO64(MB, EPI_STORE, bf16_t);                    \
     else if (out_dtype == FG_F32) GO64(MB, EPI_STORE, float);                      \
     else return FG_ERR_ARG;                                                        \

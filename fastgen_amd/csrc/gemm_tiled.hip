@@ -34,6 +34,16 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define EPI_STORE 0
 #define EPI_SILU_MUL 1
+#define EPI_GELU_MUL 4  // as EPI_SILU_MUL with another activation
+
+// silu(gate) * up, or with EPI_GELU_MUL the tanh form of GELU: 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * up
+#define EPI_IS_GATED(e) ((e) == EPI_SILU_MUL || (e) == EPI_GELU_MUL)
+template <int EPI>
+__device__ __forceinline__ float fg_gated(float gate, float up) {
+  if (EPI == EPI_GELU_MUL)
+    return 0.5f * gate * (1.f + tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate))) * up;
+  return gate / (1.f + __expf(-gate)) * up;
+}
 
 __device__ __forceinline__ bf16x8 gt_zero8() {
   bf16x8 z;
@@ -164,7 +174,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(
         for (int i = 0; i < 4; ++i) {
           const float up = __shfl_xor(acc[mb][nb][i], 32, FG_WAVE);
           const float gate = acc[mb][nb][i];
-          act[i] = gate / (1.f + __expf(-gate)) * up;
+          act[i] = fg_gated<EPI>(gate, up);
         }
         const int col = n0 / 2 + 4 * g;  // n0 is a multiple of 16: 8 channels a block
         if (g < 2 && m < M && n0 + 8 + 4 * g + 3 < N) {
@@ -217,9 +227,9 @@ extern "C" int fg_gemm_tiled(const void* x, int ldx, const void* w, int ldw, voi
   if (K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K) || k_splits < 1 || k_splits > 65535 ||
       (tile_rows != 128 && tile_rows != 256))
     return FG_ERR_ARG;
-  if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
+  if (EPI_IS_GATED(epilogue) && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && (ldy < N || (k_splits > 1 && out_dtype != FG_F32))) return FG_ERR_ARG;
-  if (epilogue != EPI_STORE && epilogue != EPI_SILU_MUL) return FG_ERR_ARG;
+  if (epilogue != EPI_STORE && !EPI_IS_GATED(epilogue)) return FG_ERR_ARG;
   if (out_dtype != FG_BF16 && out_dtype != FG_F32) return FG_ERR_ARG;
   if (((long long)M + 127) / 128 > 65535) return FG_ERR_ARG;
   const int k_per_split = ((K + k_splits * 32 - 1) / (k_splits * 32)) * 32;
@@ -228,6 +238,7 @@ extern "C" int fg_gemm_tiled(const void* x, int ldx, const void* w, int ldw, voi
 #define PICK(WM, WN, NST)                                                   \
   do {                                                                      \
     if (epilogue == EPI_SILU_MUL) GO(WM, WN, NST, EPI_SILU_MUL, bf16_t);    \
+    else if (epilogue == EPI_GELU_MUL) GO(WM, WN, NST, EPI_GELU_MUL, bf16_t); \
     else if (out_dtype == FG_BF16) GO(WM, WN, NST, EPI_STORE, bf16_t);      \
     else GO(WM, WN, NST, EPI_STORE, float);                                 \
   } while (0)

@@ -394,3 +394,140 @@ extern "C" int fg_silu_mul(const void* gu, void* out, int n_rows, int hidden, in
   }
   return fg_launch_status();
 }
+
+// ------------------------------------------- a sublayer's output, normed, then added
+// The sublayer's output d (rows of the activation dtype, or fp32 partial sums added in order) is
+// RMS-normed with the weight wp, the result is added to the fp32 stream, and, if `w` is given, the
+// stream's row is normed with `w` into `out`:
+//   h += d * rsqrt(mean(d^2) + eps_p) * wp ;  out = h * rsqrt(mean(h^2) + eps) * w
+// all in fp32 with one rounding at the store of `out`.  With `rows` only the gathered rows are
+// computed and h is left as it was.  A thread keeps its elements i = tid, tid + 256, .. in registers.
+#define POST_MAX_PER_THREAD 64  // rows of up to 16,384 elements
+template <class TA, class TW, int NIT>
+__global__ __launch_bounds__(ROWS_THREADS) void post_add_rmsnorm_kernel(
+    float* __restrict__ h, const TA* __restrict__ delta, const float* __restrict__ parts, int n_parts,
+    size_t part_stride, const TW* __restrict__ wp, float eps_p, const TW* __restrict__ w, TA* __restrict__ out,
+    const int* __restrict__ rows, int dim, float eps) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* hrow = h + src * dim;
+  float d[NIT];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NIT; ++j) {
+    const int i = threadIdx.x + j * ROWS_THREADS;
+    if (i >= dim) continue;
+    float v = 0.f;
+    if (delta) v = to_f<TA>(delta[src * dim + i]);
+    if (parts)
+      for (int p = 0; p < n_parts; ++p) v += parts[p * part_stride + src * dim + i];
+    d[j] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float rstd_p = rsqrtf(ss / (float)dim + eps_p);
+  float s2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < NIT; ++j) {
+    const int i = threadIdx.x + j * ROWS_THREADS;
+    if (i >= dim) continue;
+    const float v = hrow[i] + d[j] * rstd_p * to_f<TW>(wp[i]);
+    if (!rows) hrow[i] = v;
+    d[j] = v;
+    s2 += v * v;
+  }
+  if (!w) return;  // uniform
+  s2 = block_sum(s2, red);
+  const float rstd = rsqrtf(s2 / (float)dim + eps);
+  TA* orow = out + (size_t)r * dim;
+#pragma unroll
+  for (int j = 0; j < NIT; ++j) {
+    const int i = threadIdx.x + j * ROWS_THREADS;
+    if (i >= dim) continue;
+    orow[i] = from_f<TA>(d[j] * rstd * to_f<TW>(w[i]));
+  }
+}
+
+extern "C" int fg_post_add_rmsnorm(float* h, const void* delta, const float* parts, int n_parts,
+                                   long long part_stride, const void* wp, float eps_p, const void* w, void* out,
+                                   const int* rows, int n_rows, int dim, float eps, int act_dtype, int w_dtype,
+                                   hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (dim <= 0 || dim > POST_MAX_PER_THREAD * ROWS_THREADS || (parts && n_parts < 1) || !wp || (w && !out) ||
+      (!delta && !parts))
+    return FG_ERR_ARG;
+#define GO(TA, TW, NIT)                                                                                       \
+  post_add_rmsnorm_kernel<TA, TW, NIT><<<n_rows, ROWS_THREADS, 0, stream>>>(                                  \
+      h, (const TA*)delta, parts, n_parts, (size_t)part_stride, (const TW*)wp, eps_p, (const TW*)w, (TA*)out, \
+      rows, dim, eps)
+#define LAUNCH(TA, TW)                                 \
+  do {                                                 \
+    if (dim <= 4 * ROWS_THREADS) GO(TA, TW, 4);        \
+    else if (dim <= 16 * ROWS_THREADS) GO(TA, TW, 16); \
+    else GO(TA, TW, POST_MAX_PER_THREAD);              \
+  } while (0)
+  if (act_dtype == FG_F32 && w_dtype == FG_F32) LAUNCH(float, float);
+  else if (act_dtype == FG_BF16 && w_dtype == FG_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (act_dtype == FG_BF16 && w_dtype == FG_F32) LAUNCH(bf16_t, float);
+  else if (act_dtype == FG_F32 && w_dtype == FG_BF16) LAUNCH(float, bf16_t);
+  else return FG_ERR_ARG;
+#undef LAUNCH
+#undef GO
+  return fg_launch_status();
+}
+
+// ------------------------------------------------------ gelu_tanh(g) * u
+// As silu_mul_vec_kernel, with the tanh form of GELU: 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).
+template <class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void gelu_mul_vec_kernel(
+    const TA* __restrict__ gu, TA* __restrict__ out, int hidden) {
+  const TA* row = gu + (size_t)blockIdx.y * 2 * hidden;
+  TA* o = out + (size_t)blockIdx.y * hidden;
+  const int e = (blockIdx.x * ROWS_THREADS + threadIdx.x) * 8;
+  if (e < hidden) {
+    float gv[8], uv[8], r[8];
+    load8<TA>(row + 2 * e, gv);
+    load8<TA>(row + 2 * e + 8, uv);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float g = gv[i];
+      r[i] = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * uv[i];
+    }
+    store8<TA>(o + e, r);
+  }
+}
+
+extern "C" int fg_gelu_mul(const void* gu, void* out, int n_rows, int hidden, int act_dtype,
+                           hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (hidden <= 0 || hidden % 8 || n_rows > 65535 * 32) return FG_ERR_ARG;
+  for (int r0 = 0; r0 < n_rows; r0 += 65535) {
+    const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    const int per_block = ROWS_THREADS * 8;
+    dim3 grid((hidden + per_block - 1) / per_block, nr);
+    if (act_dtype == FG_F32)
+      gelu_mul_vec_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>((const float*)gu + (size_t)r0 * 2 * hidden,
+                                                                    (float*)out + (size_t)r0 * hidden, hidden);
+    else if (act_dtype == FG_BF16)
+      gelu_mul_vec_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const bf16_t*)gu + (size_t)r0 * 2 * hidden,
+                                                                     (bf16_t*)out + (size_t)r0 * hidden, hidden);
+    else
+      return FG_ERR_ARG;
+  }
+  return fg_launch_status();
+}
+
+// ------------------------------------------------------------- soft cap
+// x = cap * tanh(x / cap) in place on fp32 (logits).
+__global__ __launch_bounds__(ROWS_THREADS) void softcap_kernel(float* __restrict__ x, size_t n, float cap) {
+  const size_t i = (size_t)blockIdx.x * ROWS_THREADS + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" int fg_softcap(float* x, long long n, float cap, hipStream_t stream) {
+  if (n <= 0) return FG_OK;
+  if (!(cap > 0.f) || (n + ROWS_THREADS - 1) / ROWS_THREADS > 2147483647LL) return FG_ERR_ARG;
+  softcap_kernel<<<(unsigned)((n + ROWS_THREADS - 1) / ROWS_THREADS), ROWS_THREADS, 0, stream>>>(x, (size_t)n, cap);
+  return fg_launch_status();
+}

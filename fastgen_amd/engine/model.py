@@ -8,6 +8,7 @@ The reference's counterpart is the weight-only ``Transformer`` skeleton
 
 from __future__ import annotations
 
+import inspect
 import math
 from dataclasses import dataclass, field
 from pathlib import Path
@@ -17,7 +18,7 @@ import torch
 
 from ..config import ModelLayout, PartSpec, get_architecture, read_config_json
 from ..kernels.linear import StreamedMatrix, packing, packing_fits
-from ..kernels.ops import ScaledRows
+from ..kernels.ops import PostNormed, ScaledRows, post_add_rmsnorm
 from ..parts import LayerStore, PagedNeed, StateNeed, TensorSpec, build_part
 from ..parts.base import MATRIX
 from ..weights.source import RandomSource, SafetensorsSource, TensorSource, check_against_specs
@@ -83,9 +84,16 @@ class Model:
     # ------------------------------------------------------------- build
     @classmethod
     def from_config(cls, config: Mapping[str, Any], dtype: torch.dtype, device: torch.device | str,
-                    packed_weights: Optional[bool] = None, memory_budget: Optional[int] = None) -> "Model":
+                    packed_weights: Optional[bool] = None, memory_budget: Optional[int] = None,
+                    source: Optional[TensorSource] = None) -> "Model":
+        """``source``: the checkpoint, for an architecture some of whose sizes only the tensors' shapes give
+        (its ``parse`` then takes a second argument, a function from a tensor's name to its shape or None)."""
         arch = get_architecture(config)
-        args = arch.parse(config)
+        if source is not None and len(inspect.signature(arch.parse).parameters) > 1:
+            names = set(source.names())
+            args = arch.parse(config, lambda name: source.shape(name) if name in names else None)
+        else:
+            args = arch.parse(config)
         return cls(arch.layout(args), dtype, device, args=args, architecture=arch.name, packed_weights=packed_weights,
                    memory_budget=memory_budget)
 
@@ -93,8 +101,9 @@ class Model:
     def from_folder(cls, model_dir: str | Path, dtype: torch.dtype, device: torch.device | str,
                     packed_weights: Optional[bool] = None, memory_budget: Optional[int] = None) -> "Model":
         """The model that ``config.json`` names, with the folder's weights."""
-        model = cls.from_config(read_config_json(model_dir), dtype, device, packed_weights, memory_budget)
-        model.load(SafetensorsSource(model_dir))
+        source = SafetensorsSource(model_dir)
+        model = cls.from_config(read_config_json(model_dir), dtype, device, packed_weights, memory_budget, source)
+        model.load(source)
         return model
 
     @classmethod
@@ -173,6 +182,9 @@ class Model:
         for i, entry in enumerate(order):
             block = blocks[entry.layer]
             if entry.inject is not None:
+                if isinstance(pending, PostNormed):  # a sublayer's output that is normed before it is added
+                    post_add_rmsnorm(h, pending.rows, pending.weight, pending.eps, None, 0.0, None)
+                    pending = None
                 injections[entry.inject[0]].forward(h, None if isinstance(pending, ScaledRows) else pending,
                                                     embedded, entry.inject[1])
                 pending = None

@@ -45,6 +45,8 @@ LIBRARIES: Dict[str, str] = {
     "gemm_tiled": "gemm_tiled.hip",
     "sampling": "sampling.hip",
     "moe": "moe.hip",
+    "heads": "heads.hip",
+    "recurrence": "recurrence.hip",
 }
 
 # libraries compiled once per value of a macro: name -> (source, macro, values that build_all compiles,

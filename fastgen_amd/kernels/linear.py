@@ -253,16 +253,19 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None,
 
     ``epilogue="silu_mul"``: ``w`` is a gate and an up matrix interleaved by
     :func:`~fastgen_amd.kernels.ops.interleave_gate_up` and the result is
-    ``silu(gate) * up`` ``[M, N/2]``, in the product's kernel where one that does so is the fastest.
+    ``silu(gate) * up`` ``[M, N/2]``, in the product's kernel where one that does so is the fastest;
+    ``"gelu_tanh_mul"``: the same with the tanh form of GELU.
 
     ``x`` may be :class:`~fastgen_amd.kernels.ops.ScaledRows`.  ``residual`` = (h, norm weight,
     eps) asks for more than the product: add it to the fp32 residual stream ``h`` and prepare the
     RMSNorm that follows.  Where that can be folded into the product's kernel (few rows, bfloat16)
     the result is ``ScaledRows`` and ``h`` is updated; where not, the plain product comes back and
     adding and norming are the caller's."""
-    silu = epilogue == "silu_mul"
-    if epilogue not in (None, "silu_mul"):
+    silu = epilogue in ("silu_mul", "gelu_tanh_mul")  # a gated epilogue: act(gate) * up
+    if epilogue not in (None, "silu_mul", "gelu_tanh_mul"):
         raise ops.KernelArgumentError(f"linear: unknown epilogue {epilogue!r}")
+    gated = "gelu_tanh" if epilogue == "gelu_tanh_mul" else True  # what the kernels' epilogue argument takes
+    act_mul = ops.gelu_mul if epilogue == "gelu_tanh_mul" else ops.silu_mul
     sw = w.streaming if isinstance(w, StreamedMatrix) else w  # what the streaming kernels read
     w = _rows_of(w)
     scaled = x if isinstance(x, ops.ScaledRows) else None
@@ -277,7 +280,7 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None,
         if out_dtype not in (None, torch.float32):
             raise ops.KernelArgumentError("a float32 product has float32 output")
         y = ops.gemm_nt(x, w)
-        return ops.silu_mul(y) if silu else y
+        return act_mul(y) if silu else y
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
     out_dtype = out_dtype or torch.bfloat16
@@ -298,7 +301,7 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None,
             y = _library_mm_f32_out(xin, w)
             if y is None:
                 y = ops.gemm_nt(xin, w, out_dtype=torch.float32)
-        return ops.silu_mul(y) if silu else y
+        return act_mul(y) if silu else y
 
     candidates: List[Tuple[str, Callable[[], torch.Tensor]]] = []
     handicap: Dict[str, float] = {}
@@ -310,11 +313,11 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None,
 
     if own and silu and out_dtype == torch.bfloat16 and N % 16 == 0:
         if rows <= SKINNY_ROWS:
-            candidates.append(("narrow", lambda: ops.gemm_skinny(src, sw, silu_mul_epilogue=True, wide=False)))
+            candidates.append(("narrow", lambda: ops.gemm_skinny(src, sw, silu_mul_epilogue=gated, wide=False)))
         if rows <= WIDE_ROWS:
-            candidates.append(("wide", lambda: ops.gemm_skinny(src, sw, silu_mul_epilogue=True, wide=True)))
+            candidates.append(("wide", lambda: ops.gemm_skinny(src, sw, silu_mul_epilogue=gated, wide=True)))
         if tiled_ok:
-            candidates.append(("tiled256", lambda: ops.gemm_tiled(x, sw, silu_mul_epilogue=True, tile_rows=256)))
+            candidates.append(("tiled256", lambda: ops.gemm_tiled(x, sw, silu_mul_epilogue=gated, tile_rows=256)))
     elif own and not silu:
         if rows <= SKINNY_ROWS:
             candidates.append(("narrow", lambda: ops.gemm_skinny(src, sw, out_dtype, wide=False)))
@@ -332,7 +335,7 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None,
                 handicap[name] = sums_cost(s_t)
     if scaled is None or not candidates:
         candidates.append(("library", library))
-    what = ("silu_mul" if silu else "store") + ("+partials" if partials_ok and rows > SKINNY_ROWS else "") + (
+    what = (epilogue if silu else "store") + ("+partials" if partials_ok and rows > SKINNY_ROWS else "") + (
         "+f32" if out_dtype == torch.float32 else "") + ("+scaled" if scaled is not None else "") + (
         "+packed" if sw is not w else "")
     name = _choose(what, N, K, rows, candidates, handicap)

@@ -237,6 +237,71 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+def gelu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``gelu_tanh(gate) * up`` of ``[T, 2*hidden]`` laid out as :func:`silu_mul` takes it;
+    ``gelu_tanh(g) = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))``, fp32 inside."""
+    _gpu(gate_up, out)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 16 == 0,
+          "gate_up must be contiguous [T, 2*hidden] with hidden a multiple of 8")
+    T, hidden = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, hidden), dtype=gate_up.dtype, device=gate_up.device) if out is None else out
+    _need(out.shape == (T, hidden) and out.dtype == gate_up.dtype and out.is_contiguous(), "out must be [T, hidden]")
+    st = _lib.load("rows").fg_gelu_mul(_ptr(gate_up), _ptr(out), T, hidden, _code(out), _stream(out))
+    _check(st, "gelu_mul")
+    return out
+
+
+@dataclass
+class PostNormed:
+    """A sublayer's output that is RMS-normed (``weight``, ``eps``) before it is added to the residual
+    stream: ``rows`` is ``[T, dim]`` of the activation dtype or fp32 ``[S, T, dim]`` partial sums.  A norm
+    on the stream takes it where it takes rows to be added (:func:`post_add_rmsnorm`)."""
+
+    rows: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+
+
+def post_add_rmsnorm(h: torch.Tensor, delta: torch.Tensor, post_weight: torch.Tensor, post_eps: float,
+                     weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+                     rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``h += rmsnorm(delta) * post_weight`` on the fp32 stream ``h [T, dim]`` and, with ``weight``,
+    ``out = rmsnorm(h) * weight``: the norm behind a sublayer, the addition and the norm before the next
+    one in one pass, all in fp32.  ``delta`` as :func:`add_rmsnorm` takes it.  With ``rows`` only those
+    rows are computed, into consecutive rows of ``out``, and ``h`` is left as it was."""
+    _gpu(h, delta, post_weight, weight, out, rows)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [T, dim]")
+    T, dim = h.shape
+    n_rows = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, "rows")
+    _need(post_weight.shape == (dim,) and post_weight.is_contiguous(), "post_weight must be [dim]")
+    if weight is not None:
+        _need(weight.shape == (dim,) and weight.is_contiguous() and weight.dtype == post_weight.dtype,
+              "weight must be [dim], of post_weight's dtype")
+        _need(out is not None and out.is_contiguous() and out.shape == (n_rows, dim), "out must be contiguous [rows, dim]")
+    else:
+        _need(rows is None, "a gathered call computes the norm that follows")
+    act = out.dtype if out is not None else (delta.dtype if delta.dim() == 2 else torch.float32)
+    d_ptr, d_code, parts, n_parts, part_stride = _delta_args(h, delta, "post_add_rmsnorm")
+    if delta.dim() == 2:
+        _need(delta.dtype == act, "delta must have out's dtype")
+    st = _lib.load("rows").fg_post_add_rmsnorm(
+        _ptr(h), d_ptr, parts, n_parts, part_stride, _ptr(post_weight), ctypes.c_float(post_eps), _ptr(weight),
+        _ptr(out), _ptr(rows), n_rows, dim, ctypes.c_float(eps), _DTYPE_CODE[act], _code(post_weight), _stream(h))
+    _check(st, "post_add_rmsnorm")
+    return out
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x = cap * tanh(x / cap)`` in place on contiguous fp32."""
+    _gpu(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and cap > 0, "x must be contiguous float32, cap positive")
+    st = _lib.load("rows").fg_softcap(_ptr(x), ctypes.c_longlong(x.numel()), ctypes.c_float(cap), _stream(x))
+    _check(st, "softcap")
+    return x
+
+
 # ------------------------------------------------------------ rope + kv write
 def rope_table(positions: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
     """``[T, n_freqs, 2]`` fp32: cos and sin of ``float(pos) * freqs[i]``, for all
@@ -297,15 +362,25 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[to
 
 
 # ------------------------------------------------------------------ attention
+def _sinks_ok(sinks: Optional[torch.Tensor], n_heads: int) -> None:
+    if sinks is not None:
+        _need(sinks.dtype == torch.float32 and sinks.is_contiguous() and sinks.shape == (n_heads,),
+              "sinks must be contiguous float32 [n_heads]")
+
+
 def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                             block_table: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
-                            n_heads: int, scale: float, window: int = 0) -> torch.Tensor:
+                            n_heads: int, scale: float, window: int = 0,
+                            sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of every token over its sequence's cached keys.
 
     ``q`` is ``[T, >= H*hd]`` (the first ``H*hd`` columns are the query heads;
     it may be a qkv buffer), ``out`` is ``[T, H*hd]``.  ``forward.py:176-258``.
+    ``sinks``: fp32 ``[H]``; head ``h``'s softmax has one more term ``exp(sinks[h])`` in its
+    denominator, which brings no value.
     """
-    _gpu(q, out, k_pages, v_pages, block_table, seq_of_token, positions)
+    _gpu(q, out, k_pages, v_pages, block_table, seq_of_token, positions, sinks)
+    _sinks_ok(sinks, n_heads)
     T = q.shape[0]
     _need(k_pages.dim() == 4 and k_pages.is_contiguous(), "k_pages must be contiguous [n_pages, KV, P, hd]")
     n_pages, n_kv, page_size, hd = k_pages.shape
@@ -321,10 +396,10 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
     _need(n_heads % n_kv == 0, "the number of heads must be a multiple of the number of kv heads")
     _need(hd % 8 == 0 and hd <= 512, f"head size {hd} is not supported (multiple of 8, at most 512)")
     _need(page_size % 8 == 0, f"page size {page_size} is not supported (multiple of 8)")
-    st = _lib.load("attention").fg_paged_attention_general(
+    st = _lib.load("attention").fg_paged_attention_general_sink(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         block_table.stride(0), _ptr(seq_of_token), _ptr(positions), T, n_heads, n_kv, hd, page_size,
-        ctypes.c_float(scale), int(window or 0), _code(q), _stream(q))
+        ctypes.c_float(scale), int(window or 0), _ptr(sinks), _code(q), _stream(q))
     _check(st, "paged_attention_general")
     return out
 
@@ -436,7 +511,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
                          plan: Optional[torch.Tensor] = None, max_chunks: Optional[int] = None,
                          min_tiles: int = 4, max_rows: int = 16, tile_rows: Optional[int] = None,
-                         exact_weights: bool = False) -> torch.Tensor:
+                         exact_weights: bool = False, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``small_items`` / ``big_items`` are
     device int32 ``[n, 4]`` lists from :func:`attention_items` (16-byte aligned);
     every query token of the step must be covered by exactly one item.
@@ -447,8 +522,10 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
     With items of both kinds the tile kernel runs on a second stream beside the split kernel and
     the current stream waits for it before this returns (not while a graph is captured, not with
     ``FG_ONE_STREAM=1``).  ``exact_weights``: the build of the kernels in which the softmax weights enter
-    the product with the values as two bfloat16 terms (16 significant bits)."""
-    _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items, plan)
+    the product with the values as two bfloat16 terms (16 significant bits).  ``sinks``: as
+    :func:`paged_attention_general`."""
+    _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items, plan, sinks)
+    _sinks_ok(sinks, n_heads)
     n_pages, n_kv, page_size, hd = k_pages.shape
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
           and v_pages.dtype == torch.bfloat16, "the MFMA attention kernels take bfloat16")
@@ -487,10 +564,10 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
               "the plan does not fit the items and max_chunks")
         part_o = torch.empty((max_chunks * n_kv * 16, hd), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((max_chunks * n_kv * 16, 2), dtype=torch.float32, device=q.device)
-        st = lib.fg_attn_split(
+        st = lib.fg_attn_split_sink(
             _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.stride(0), _ptr(plan), n, max_chunks, max_rows, _ptr(part_o), _ptr(part_ml), n_heads, n_kv, hd,
-            page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
+            page_size, ctypes.c_float(scale), int(window or 0), _ptr(sinks), _stream(q))
         _check(st, "attn_split")
     if big_items is not None and big_items.numel():
         tile_rows = attention_tile_rows(hd, False, exact_weights) if tile_rows is None else int(tile_rows)
@@ -499,10 +576,11 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
         _need(G <= tile_rows, "too many query heads per kv head for the tile kernel")
         _i32(big_items, "big_items")
         _need(big_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
-        st = lib.fg_attn_tile(
+        st = lib.fg_attn_tile_sink(
             _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.stride(0), _ptr(big_items), big_items.numel() // 4, tile_rows, n_heads, n_kv, hd, page_size,
-            ctypes.c_float(scale), int(window or 0), ctypes.c_void_p(beside.cuda_stream) if beside else _stream(q))
+            ctypes.c_float(scale), int(window or 0), _ptr(sinks),
+            ctypes.c_void_p(beside.cuda_stream) if beside else _stream(q))
         _check(st, "attn_tile")
         if beside is not None:
             torch.cuda.current_stream(q.device).wait_event(beside.record_event())
@@ -511,7 +589,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                     group, ctx, n_heads: int, scale: float, window: int = 0,
-                    exact_weights: bool = False) -> torch.Tensor:
+                    exact_weights: bool = False, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention for one step: picks the kernel for the step's dtype and shape.
     ``exact_weights``: see :func:`paged_attention_mfma` (the general kernel's weights are fp32 anyway).
 
@@ -525,7 +603,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
     G = n_heads // n_kv
     if q.dtype != torch.bfloat16 or hd % 16 or hd > MFMA_MAX_HEAD_DIM or G > 16:
         return paged_attention_general(q, out, k_pages, v_pages, group.block_table, ctx.seq_of_token,
-                                       ctx.positions, n_heads, scale, window)
+                                       ctx.positions, n_heads, scale, window, sinks)
     items_key = ("attention_items", G, hd, n_kv)  # (how a step is cut into items depends on all three)
     plan = ctx.scratch.get(items_key)
     if plan is None:
@@ -560,7 +638,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
     rows = G * int(ctx.q_lens.max()) if big_d is None else 16
     return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
                                 window, split_plan, chunks, max_rows=min(16, rows), tile_rows=tile_rows,
-                                exact_weights=exact_weights)
+                                exact_weights=exact_weights, sinks=sinks)
 
 
 # ----------------------------------------------------------------------- gemm
@@ -587,6 +665,17 @@ def gemm_nt(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None
 
 
 SKINNY_MAX_ROWS = 128
+
+# epilogue codes of the streaming and tiled products: store; silu(gate) * up; gelu_tanh(gate) * up
+_GATED_CODE = {False: 0, None: 0, True: 1, "silu": 1, "gelu_tanh": 4}
+
+
+def _gated_code(epilogue) -> int:
+    """The kernels' code for a ``silu_mul_epilogue`` argument: False, True (SiLU), or the activation's name."""
+    try:
+        return _GATED_CODE[epilogue]
+    except (KeyError, TypeError):
+        raise KernelArgumentError(f"unknown gated epilogue {epilogue!r} (True, 'silu' or 'gelu_tanh')") from None
 
 
 @dataclass
@@ -731,7 +820,7 @@ def gemm_skinny(x, w, out_dtype: Optional[torch.dtype] = None,
     stream ``w [N, K]`` (a matrix or :class:`PackedWeight`) once.  ``x`` may be :class:`ScaledRows` (at most 16 rows, bfloat16 out): the
     result rows are scaled.  With ``silu_mul_epilogue`` ``w`` is a gate/up matrix
     ordered by :func:`interleave_gate_up` and the result is ``silu(gate) * up``
-    ``[M, N/2]``.  With ``k_splits > 1`` the k range is cut over workgroups and the
+    ``[M, N/2]`` (``"gelu_tanh"`` in True's place: that activation in SiLU's).  With ``k_splits > 1`` the k range is cut over workgroups and the
     result is fp32 ``[k_splits, M, N]`` partial sums (for few output columns,
     where one workgroup per 64 columns would leave most of the GPU idle).
     ``wide`` picks the kernel for 17..128 rows (64 columns a workgroup, x shared
@@ -762,21 +851,21 @@ def gemm_skinny(x, w, out_dtype: Optional[torch.dtype] = None,
         _need(M <= 16 and k_splits == 1 and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
         st = lib.fg_gemm_skinny64(
             _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), cols, ctypes.c_longlong(M * cols), 1, M, N,
-            K, _code(y), 1 if silu_mul_epilogue else 0, *_row_scale_args(scaled, M), _stream(x))
+            K, _code(y), _gated_code(silu_mul_epilogue), *_row_scale_args(scaled, M), _stream(x))
     elif scaled is not None:
         _need(M <= 16 and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
         st = lib.fg_gemm_skinny_fused(
-            _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), y.stride(0), M, N, K, 1 if silu_mul_epilogue else 0,
+            _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), y.stride(0), M, N, K, _gated_code(silu_mul_epilogue),
             *_row_scale_args(scaled, M), ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0,
             ctypes.c_void_p(0), _stream(x))
     elif wide:
         st = lib.fg_gemm_skinny64(
             _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N,
-            K, _code(y), 1 if silu_mul_epilogue else 0, *_row_scale_args(None, M), _stream(x))
+            K, _code(y), _gated_code(silu_mul_epilogue), *_row_scale_args(None, M), _stream(x))
     else:
         st = lib.fg_gemm_skinny(
             _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), y.stride(0), M, N, K, _code(y),
-            1 if silu_mul_epilogue else 0, _stream(x))
+            _gated_code(silu_mul_epilogue), _stream(x))
     _check(st, "gemm_skinny")
     return y
 
@@ -809,7 +898,7 @@ def gemm_tiled(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None,
     y = torch.empty((k_splits, M, cols) if k_splits > 1 else (M, cols), dtype=out_dtype, device=x.device)
     st = _lib.load("gemm_tiled").fg_gemm_tiled(
         _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N, K,
-        _code(y), 1 if silu_mul_epilogue else 0, int(tile_rows), _stream(x))
+        _code(y), _gated_code(silu_mul_epilogue), int(tile_rows), _stream(x))
     _check(st, "gemm_tiled")
     return y
 
@@ -1015,4 +1104,196 @@ def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tens
     st = _lib.load("moe").fg_moe_combine(_ptr(y), _ptr(weight), _ptr(plus), ldp, _code(plus) if plus is not None else F32,
                                          n_plus, ctypes.c_longlong(stride), T, top, dim, _ptr(out), _stream(y))
     _check(st, "moe_combine")
+    return out
+
+
+# ------------------------------------------------------------- per-head work
+class _PrepareArgs(ctypes.Structure):
+    _fields_ = [("src", ctypes.c_void_p), ("src_stride", ctypes.c_int), ("bias", ctypes.c_void_p),
+                ("n_q", ctypes.c_int), ("q_col", ctypes.c_int), ("q_w", ctypes.c_int), ("q_norm_dims", ctypes.c_int),
+                ("q_norm_w", ctypes.c_void_p), ("q_out", ctypes.c_void_p), ("q_out_stride", ctypes.c_int),
+                ("q_out_hw", ctypes.c_int), ("n_kv", ctypes.c_int), ("k_col", ctypes.c_int), ("k_w", ctypes.c_int),
+                ("k_norm_dims", ctypes.c_int), ("k_norm_w", ctypes.c_void_p), ("v_col", ctypes.c_int),
+                ("v_w", ctypes.c_int), ("table", ctypes.c_void_p), ("rot_start", ctypes.c_int),
+                ("rotary_dim", ctypes.c_int), ("rot_q", ctypes.c_int), ("rot_k", ctypes.c_int), ("eps", ctypes.c_float), ("slots", ctypes.c_void_p),
+                ("k_pages", ctypes.c_void_p), ("v_pages", ctypes.c_void_p), ("page_size", ctypes.c_int),
+                ("hd_c", ctypes.c_int)]
+
+
+def _f32_vec(t: Optional[torch.Tensor], n: int, name: str) -> None:
+    if t is not None:
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n, f"{name} must be contiguous float32 [{n}]")
+
+
+def heads_prepare(src: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                  n_q: int = 0, q_col: int = 0, q_width: int = 0, q_norm: Optional[torch.Tensor] = None,
+                  q_norm_dims: int = 0, q_out: Optional[torch.Tensor] = None, q_out_width: int = 0,
+                  n_kv: int = 0, k_col: int = 0, k_width: int = 0, k_norm: Optional[torch.Tensor] = None,
+                  k_norm_dims: int = 0, v_col: int = -1, v_width: int = 0,
+                  table: Optional[torch.Tensor] = None, rot_start: int = 0, rotary_dim: int = 0,
+                  rotate_q: bool = True, rotate_k: bool = True, slots: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
+                  v_pages: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """What lies between a product's rows ``src [T, width]`` (fp32, or the activation dtype) and an attention.
+
+    Per token and head: add ``bias`` (fp32, per column of ``src``); RMS-norm the head's first ``*_norm_dims``
+    elements with the fp32 weight ``*_norm`` (if given) and ``eps``; turn the pairs
+    ``(rot_start + 2i, rot_start + 2i + 1)``, ``i < rotary_dim / 2``, by the angles of ``table``
+    (:func:`rope_table`; ``rotate_q`` / ``rotate_k``: whether query and key heads turn).  The ``n_q`` query heads (``q_width`` wide, from column ``q_col``) go to
+    ``q_out [T, n_q * q_out_width]`` of the cache's dtype, each padded with zeros to ``q_out_width``.
+    The ``n_kv`` key heads (``k_width`` wide, from ``k_col``) go to ``slots`` of ``k_pages
+    [n_pages, n_kv, P, hd]`` padded with zeros to ``hd``; the values (``v_width`` wide) to ``v_pages
+    [n_pages, n_kv, hd, P]`` likewise: columns of their own from ``v_col``, with their bias, or, with
+    ``v_col < 0``, the first ``v_width`` elements of the processed key.  A negative slot writes nothing."""
+    _gpu(src, bias, q_norm, q_out, k_norm, table, slots, k_pages, v_pages)
+    _need(src.dim() == 2 and src.stride(1) == 1, "src must be [T, width] with unit column stride")
+    T, width = src.shape
+    a = _PrepareArgs()
+    a.src, a.src_stride, a.bias, a.eps = src.data_ptr(), src.stride(0), bias.data_ptr() if bias is not None else None, eps
+    _f32_vec(bias, width, "bias")
+    act = None
+    a.n_q, a.n_kv = int(n_q), int(n_kv)
+    _need(n_q >= 0 and n_kv >= 0 and n_q + n_kv > 0, "there must be heads to prepare")
+    if n_q:
+        _need(q_out is not None and q_out.dim() == 2 and q_out.stride(1) == 1 and q_out.shape[0] == T
+              and q_out.shape[1] >= n_q * q_out_width and q_out_width >= q_width > 0,
+              "q_out must be [T, >= n_q * q_out_width] with q_out_width >= q_width")
+        _need(q_col >= 0 and q_col + n_q * q_width <= width, "the query heads lie outside src")
+        _need(q_width % 2 == 0 and q_out_width % 2 == 0 and q_out_width <= 1024, "head widths must be even, at most 1024")
+        _need(0 <= q_norm_dims <= q_width and q_norm_dims % 2 == 0, "q_norm_dims must be even and at most q_width")
+        _f32_vec(q_norm, q_norm_dims, "q_norm")
+        _need(q_norm is None or q_norm_dims > 0, "a norm needs dimensions to run over")
+        act = q_out.dtype
+        a.q_col, a.q_w, a.q_norm_dims, a.q_norm_w = q_col, q_width, q_norm_dims, q_norm.data_ptr() if q_norm is not None else None
+        a.q_out, a.q_out_stride, a.q_out_hw = q_out.data_ptr(), q_out.stride(0), q_out_width
+    if n_kv:
+        _need(slots is not None and k_pages is not None and v_pages is not None, "cache operands missing")
+        _i32(slots, "slots", T)
+        _need(k_pages.dim() == 4 and k_pages.is_contiguous() and k_pages.shape[1] == n_kv, "k_pages must be contiguous [n_pages, n_kv, P, hd]")
+        n_pages, _, P, hd = k_pages.shape
+        _need(v_pages.is_contiguous() and v_pages.shape == (n_pages, n_kv, hd, P) and v_pages.dtype == k_pages.dtype,
+              "v_pages must be contiguous [n_pages, n_kv, hd, P] of k_pages' dtype")
+        _need(act is None or act == k_pages.dtype, "q_out and the cache must share a dtype")
+        act = k_pages.dtype
+        _need(P % 8 == 0 and hd % 8 == 0 and hd <= 1024, "pages of a multiple of 8 tokens, head size a multiple of 8 up to 1024")
+        _need(0 < k_width <= hd and k_width % 2 == 0 and 0 < v_width <= hd and v_width % 2 == 0,
+              "key and value widths must be even and at most the cache's head size")
+        _need(k_col >= 0 and k_col + n_kv * k_width <= width, "the key heads lie outside src")
+        _need(v_col < 0 and v_width <= k_width or v_col >= 0 and v_col + n_kv * v_width <= width,
+              "the values lie outside src (or, taken from the keys, are wider than they)")
+        _need(0 <= k_norm_dims <= k_width and k_norm_dims % 2 == 0, "k_norm_dims must be even and at most k_width")
+        _f32_vec(k_norm, k_norm_dims, "k_norm")
+        _need(k_norm is None or k_norm_dims > 0, "a norm needs dimensions to run over")
+        a.k_col, a.k_w, a.k_norm_dims, a.k_norm_w = k_col, k_width, k_norm_dims, k_norm.data_ptr() if k_norm is not None else None
+        a.v_col, a.v_w = (v_col if v_col >= 0 else -1), v_width
+        a.slots, a.k_pages, a.v_pages, a.page_size, a.hd_c = slots.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), P, hd
+    if table is not None and rotary_dim:
+        _need(table.dtype == torch.float32 and table.is_contiguous() and table.shape == (T, rotary_dim // 2, 2),
+              "table must be float32 [T, rotary_dim/2, 2]")
+        _need(rot_start >= 0 and rot_start % 2 == 0 and rotary_dim % 2 == 0, "the rotated run starts and ends at even dimensions")
+        _need((not (n_q and rotate_q) or rot_start + rotary_dim <= q_width)
+              and (not (n_kv and rotate_k) or rot_start + rotary_dim <= k_width), "the rotated run lies outside a head")
+        a.table, a.rot_start, a.rotary_dim = table.data_ptr(), rot_start, rotary_dim
+        a.rot_q, a.rot_k = int(bool(rotate_q)), int(bool(rotate_k))
+    _need(src.dtype == torch.float32 or src.dtype == act, "src must be float32 or of the cache's dtype")
+    st = _lib.load("heads").fg_heads_prepare(ctypes.byref(a), T, _code(src), _DTYPE_CODE[act], _stream(src))
+    _check(st, "heads_prepare")
+    return q_out
+
+
+class _HeadLinearArgs(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_void_p), ("x_stride", ctypes.c_int), ("x_hs", ctypes.c_int), ("w", ctypes.c_void_p),
+                ("y", ctypes.c_void_p), ("y_stride", ctypes.c_int), ("y_hs", ctypes.c_int), ("gate", ctypes.c_void_p),
+                ("gate_stride", ctypes.c_int), ("T", ctypes.c_int), ("H", ctypes.c_int), ("N", ctypes.c_int),
+                ("K", ctypes.c_int), ("tail", ctypes.c_int), ("y_hw", ctypes.c_int)]
+
+
+def head_linear(x: torch.Tensor, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_head_stride: int,
+                tail: int = 0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A product per head: ``out[t, h * out_head_stride + n] = sum_k w[h, n, k] * x[t, h * x_head_stride + k]``
+    for ``w [H, N, K]``; with fp32 ``gate [T, >= H]`` (unit column stride) the result is multiplied by
+    ``sigmoid(gate[t, h])``.  The ``tail`` columns of ``x``'s head behind ``K`` are copied behind the ``N``
+    results, and what is left of the ``out_head_stride`` columns is set to zero."""
+    _gpu(x, w, out, gate)
+    _need(w.dim() == 3 and w.is_contiguous(), "w must be contiguous [H, N, K]")
+    H, N, K = w.shape
+    T = x.shape[0]
+    _need(x.dim() == 2 and x.stride(1) == 1 and x_head_stride >= K + tail and x.shape[1] >= (H - 1) * x_head_stride + K + tail,
+          "x must be [T, >= H * x_head_stride] with heads at least K + tail wide")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == T and out_head_stride >= N + tail
+          and out.shape[1] >= H * out_head_stride, "out must be [T, >= H * out_head_stride] with heads at least N + tail wide")
+    _need(x.dtype == w.dtype == out.dtype, "x, w and out must share a dtype")
+    a = _HeadLinearArgs()
+    a.x, a.x_stride, a.x_hs, a.w = x.data_ptr(), x.stride(0), x_head_stride, w.data_ptr()
+    a.y, a.y_stride, a.y_hs = out.data_ptr(), out.stride(0), out_head_stride
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == T and gate.shape[1] >= H
+              and gate.dtype == torch.float32, "gate must be float32 [T, >= H]")
+        a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
+    a.T, a.H, a.N, a.K, a.tail, a.y_hw = T, H, N, K, tail, out_head_stride
+    mfma = (x.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(0) % 8 == 0 and x_head_stride % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    _need(mfma or K <= 1024, "heads of more than 1024 inputs need bfloat16 rows aligned to 16 bytes")
+    st = _lib.load("heads").fg_head_linear(ctypes.byref(a), _code(x), int(mfma), _stream(x))
+    _check(st, "head_linear")
+    return out
+
+
+def head_norm_gate(x: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor, n_heads: int,
+                   out: torch.Tensor) -> torch.Tensor:
+    """``out[t, h, :] = rmsnorm(x[t, h, :]) * weight * silu(gate[t, h, :])`` for fp32 ``x [T, H*e]``, fp32
+    ``weight [e]`` shared by the heads, ``gate [T, >= H*e]`` (unit column stride) and ``out [T, H*e]`` of the
+    activation dtype."""
+    _gpu(x, weight, gate, out)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and x.shape[1] % n_heads == 0, "x must be contiguous float32 [T, H*e]")
+    T, e = x.shape[0], x.shape[1] // n_heads
+    _f32_vec(weight, e, "weight")
+    _need(e <= 1024, "heads of at most 1024 elements")
+    _need(out.shape == x.shape and out.is_contiguous(), "out must be contiguous [T, H*e]")
+    _need(gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == T and gate.shape[1] >= n_heads * e
+          and gate.dtype == out.dtype, "gate must be [T, >= H*e] of out's dtype")
+    st = _lib.load("heads").fg_head_norm_gate(_ptr(x), _ptr(weight), _ptr(gate), gate.stride(0), _ptr(out), T, n_heads,
+                                              e, ctypes.c_float(eps), _code(out), _stream(out))
+    _check(st, "head_norm_gate")
+    return out
+
+
+# ---------------------------------------------------------------- recurrence
+class _ScanArgs(ctypes.Structure):
+    _fields_ = [("qkv", ctypes.c_void_p), ("row_stride", ctypes.c_int), ("q_col", ctypes.c_int), ("k_col", ctypes.c_int),
+                ("v_col", ctypes.c_int), ("z", ctypes.c_void_p), ("z_stride", ctypes.c_int), ("z_bias", ctypes.c_void_p),
+                ("inv_tau", ctypes.c_float), ("q_scale", ctypes.c_float), ("state", ctypes.c_void_p),
+                ("slot_ids", ctypes.c_void_p), ("q_start", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("H", ctypes.c_int), ("d", ctypes.c_int), ("e", ctypes.c_int)]
+
+
+def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: Optional[torch.Tensor],
+               tau: float, q_scale: float, state: torch.Tensor, slot_ids: torch.Tensor, q_start: torch.Tensor,
+               n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+    """The recurrence ``S <- diag(a_t) S + k_t v_t^T``, ``o_t = S^T (q_t * q_scale)`` with
+    ``a_t = sigmoid(z_t + z_bias)^(1/tau)``, token by token for every sequence of the step.
+
+    ``qkv [T, width]`` holds per token ``q`` and ``k`` (``H*d`` columns from ``q_col`` / ``k_col``) and ``v``
+    (``H*e`` from ``v_col``); ``z`` is fp32 ``[T, >= H*d]``; ``state`` fp32 ``[n_slots, H, d, e]`` is read at
+    ``slot_ids[b]`` and left as the sequence's last token leaves it; sequence ``b`` has the tokens
+    ``q_start[b] .. q_start[b+1]-1``; ``out`` is fp32 ``[T, H*e]``."""
+    _gpu(qkv, z, z_bias, state, slot_ids, q_start, out)
+    _need(state.dtype == torch.float32 and state.dim() == 4 and state.is_contiguous(), "state must be contiguous float32 [n_slots, H, d, e]")
+    _, H, d, e = state.shape
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and max(q_col, k_col) + H * d <= qkv.shape[1] and v_col + H * e <= qkv.shape[1]
+          and min(q_col, k_col, v_col) >= 0, "q, k and v must lie inside the rows of qkv")
+    _need(z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1 and z.shape[0] == T and z.shape[1] >= H * d,
+          "z must be float32 [T, >= H*d]")
+    _f32_vec(z_bias, H * d, "z_bias")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, H * e), "out must be contiguous float32 [T, H*e]")
+    _i32(slot_ids, "slot_ids", n_seqs)
+    _i32(q_start, "q_start", n_seqs + 1)
+    _need(d <= 256 and tau > 0, "at most 256 key channels a head; tau positive")
+    a = _ScanArgs()
+    a.qkv, a.row_stride, a.q_col, a.k_col, a.v_col = qkv.data_ptr(), qkv.stride(0), q_col, k_col, v_col
+    a.z, a.z_stride, a.z_bias = z.data_ptr(), z.stride(0), z_bias.data_ptr() if z_bias is not None else None
+    a.inv_tau, a.q_scale, a.state = 1.0 / tau, q_scale, state.data_ptr()
+    a.slot_ids, a.q_start, a.out, a.H, a.d, a.e = slot_ids.data_ptr(), q_start.data_ptr(), out.data_ptr(), H, d, e
+    st = _lib.load("recurrence").fg_decay_scan(ctypes.byref(a), int(n_seqs), _code(qkv), _stream(qkv))
+    _check(st, "decay_scan")
     return out

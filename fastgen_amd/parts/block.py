@@ -84,3 +84,36 @@ class ParallelBlock:
 
 
 register_part("arrangement", "parallel", lambda spec, *parts: ParallelBlock(*parts))
+
+
+class SandwichBlock:
+    """``h += post_mixer(mixer(norm(h))); h += post_ffn(ffn(norm(h)))``: a norm before and a norm behind every
+    sublayer.  The norms behind are ``extra_norms`` of the layer, ``post_mixer`` and ``post_ffn``.  A
+    sublayer's output goes on as :class:`~fastgen_amd.kernels.ops.PostNormed`: the norm that follows (this
+    block's second, the next block's first, the model's last) norms it, adds it to the stream and norms
+    the stream in one kernel, in fp32.  A layer without a feed-forward has only the first half."""
+
+    folds_norms = False
+
+    def __init__(self, mixer: Mixer, ffn: Optional[FeedForward], mixer_norm: Norm, ffn_norm: Optional[Norm],
+                 extra: Optional[dict] = None) -> None:
+        extra = extra or {}
+        if "post_mixer" not in extra or (ffn is not None and ("post_ffn" not in extra or ffn_norm is None)):
+            raise ValueError("a sandwich layer needs the norms post_mixer and, with a feed-forward, ffn_norm and post_ffn")
+        self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+        self.post_mixer, self.post_ffn = extra["post_mixer"], extra.get("post_ffn")
+
+    @staticmethod
+    def _behind(rows, norm) -> ops.PostNormed:
+        return ops.PostNormed(rows, norm.weight, norm.eps)
+
+    def forward(self, h: torch.Tensor, pending, ctx: Any, store: LayerStore):
+        x = self.mixer_norm.forward(h, pending, ctx.act_dtype)
+        mixed = self._behind(self.mixer.forward(x, ctx, store), self.post_mixer)
+        if self.ffn is None:
+            return mixed
+        x = self.ffn_norm.forward(h, mixed, ctx.act_dtype)
+        return self._behind(self.ffn.forward(x), self.post_ffn)
+
+
+register_part("arrangement", "sandwich", lambda spec, *parts: SandwichBlock(*parts))

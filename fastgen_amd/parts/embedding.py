@@ -37,13 +37,15 @@ class Embedding(Part):
 
 class LMHead(Part):
     """fp32 logits ``x W^T``; ``W`` is the head's own matrix or, when tied,
-    the embedding table (``fastgen/forward.py:507-515``)."""
+    the embedding table (``fastgen/forward.py:507-515``).  With the option ``softcap`` the logits are
+    ``cap * tanh(logits / cap)``."""
 
     def __init__(self, spec) -> None:
         super().__init__(spec)
         self.vocab_size = int(spec.options["vocab_size"])
         self.dim = int(spec.options["dim"])
         self.tied_to: Optional[str] = spec.options.get("tied_to")
+        self.softcap = float(spec.options.get("softcap") or 0.0)
         self.weight: Optional[StreamedMatrix] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -63,7 +65,8 @@ class LMHead(Part):
         self.weight = streamed(table)  # the table itself row by row; a packed copy of it if copies are made
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return linear(x, self.weight, out_dtype=torch.float32)
+        logits = linear(x, self.weight, out_dtype=torch.float32)
+        return ops.softcap(logits, self.softcap) if self.softcap > 0 else logits
 
 
 register_part("embedding", "embedding", Embedding)

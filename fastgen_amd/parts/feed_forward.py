@@ -2,7 +2,8 @@
 ``down(silu(gate(x)) * up(x))``.  Gate and up are one matrix with their rows
 interleaved in groups of 8, so one product gives both and a tile of it holds
 both halves of a channel: for few rows ``silu(gate) * up`` is applied where the
-product is stored."""
+product is stored.  The option ``activation`` puts the tanh form of GELU
+(``"gelu_tanh"``) in SiLU's place."""
 
 from __future__ import annotations
 
@@ -22,6 +23,9 @@ class SwiGLU(FeedForward):
         super().__init__(spec)
         self.dim = int(spec.options["dim"])
         self.hidden_dim = int(spec.options["hidden_dim"])
+        self.activation = spec.options.get("activation", "silu")
+        if self.activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"{self.prefix}: activation {self.activation!r} is not supported ('silu', 'gelu_tanh')")
         self.w_gate_up: Optional[StreamedMatrix] = None
         self.w_down: Optional[StreamedMatrix] = None
 
@@ -48,7 +52,7 @@ class SwiGLU(FeedForward):
     def forward(self, x, then=None):
         """``x``: the normed rows, or ``ScaledRows`` (the gate/up product finishes the norm).  ``then``:
         a norm's ``fold_request`` for the down projection (see ``Attention.forward``)."""
-        act = linear(x, self.w_gate_up, epilogue="silu_mul")
+        act = linear(x, self.w_gate_up, epilogue=f"{self.activation}_mul")
         return linear(act, self.w_down, partials_ok=True, residual=then)
 
 

@@ -36,8 +36,13 @@ class RMSNorm(Norm):
         return (h, self.weight, self.eps)
 
     def forward(self, h, delta, dtype, rows=None):
+        """``delta`` may be :class:`~fastgen_amd.kernels.ops.PostNormed`: a sublayer's output that is normed
+        itself before it is added (the norm behind a sublayer); one kernel does that norm, the addition and
+        this norm."""
         n = h.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.dim), dtype=dtype, device=h.device)
+        if isinstance(delta, ops.PostNormed):
+            return ops.post_add_rmsnorm(h, delta.rows, delta.weight, delta.eps, self.weight, self.eps, out, rows)
         return ops.add_rmsnorm(h, delta, self.weight, self.eps, out, rows)
 
 
