@@ -238,7 +238,8 @@ class ModelRunner:
     def _graph_for(self, entries: Sequence[StepEntry]) -> _DecodeGraph:
         """The captured step for these entries (whose pages are reserved): by batch capacity and
         block-table width.  At most ``max_graphs`` are kept; the one unused longest gives way."""
-        held = max(self.cache.n_table_entries(e.rid, g) for e in entries for g in range(self.cache.n_groups))
+        # (a model whose mixers keep state only has no cache group and no block table)
+        held = max((self.cache.n_table_entries(e.rid, g) for e in entries for g in range(self.cache.n_groups)), default=0)
         key = (self.graph_capacity(len(entries)), graph_table_width_for(held, self.table_width))
         g = self.graphs.pop(key, None)
         if g is None:

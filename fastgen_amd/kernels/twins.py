@@ -18,7 +18,7 @@ from typing import Optional
 import torch
 
 from ..cache.layout import store_k, store_v, unpack_k, unpack_v
-from .ops import PackedWeight, ScaledRows
+from .ops import PackedWeight, PostNormed, ScaledRows  # noqa: F401
 
 
 def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
@@ -104,6 +104,51 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+def _gelu_tanh(g: torch.Tensor) -> torch.Tensor:
+    return 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+
+
+def _gated(y: torch.Tensor, epilogue) -> torch.Tensor:
+    """``act(gate) * up`` of fp32 ``[M, 2F]`` interleaved in turns of 8; ``epilogue``: True or "silu", or "gelu_tanh"."""
+    M, N = y.shape
+    gu = y.view(M, N // 16, 2, 8)
+    g, u = gu[:, :, 0].reshape(M, N // 2), gu[:, :, 1].reshape(M, N // 2)
+    return (_gelu_tanh(g) if epilogue == "gelu_tanh" else g * torch.sigmoid(g)) * u
+
+
+def gelu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``gelu_tanh(gate) * up`` of ``[T, 2F]`` whose columns are interleaved in turns of 8 as above."""
+    y = _gated(gate_up.float(), "gelu_tanh").to(gate_up.dtype)
+    if out is None:
+        return y
+    out.copy_(y)
+    return out
+
+
+def post_add_rmsnorm(h: torch.Tensor, delta: torch.Tensor, post_weight: torch.Tensor, post_eps: float,
+                     weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+                     rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``h += rmsnorm(delta) * post_weight``; with ``weight``: ``out = rmsnorm(h) * weight``.  With ``rows`` only those
+    rows, into consecutive rows of ``out``, and ``h`` stays."""
+    d = sum(_added(delta))
+    d = d * torch.rsqrt((d * d).mean(-1, keepdim=True) + post_eps) * post_weight.float()
+    s = h + d
+    if rows is None:
+        h.copy_(s)
+    else:
+        s = s[rows.long()]
+    if weight is None:
+        return out
+    out.copy_((s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * weight.float()).to(out.dtype))
+    return out
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x = cap * tanh(x / cap)`` in place."""
+    x.copy_(cap * torch.tanh(x / cap))
+    return x
+
+
 def rope_table(positions: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
     """fp32 ``[T, len(freqs), 2]``: cos and sin of ``position * frequency``."""
     ang = positions.to(torch.float32)[:, None] * freqs.float()[None, :]
@@ -164,10 +209,12 @@ def _gather_kv(pages: torch.Tensor, unpack, table_row: torch.Tensor, n: int) -> 
 
 def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                             block_table: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
-                            n_heads: int, scale: float, window: int = 0) -> torch.Tensor:
+                            n_heads: int, scale: float, window: int = 0,
+                            sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Token ``t`` of sequence ``b`` at position ``p`` attends keys ``0..p`` (``p-window+1..p`` with a window)
     of its sequence, read through ``block_table[b]``; query head ``h`` reads kv head ``h // (H / KV)``;
-    softmax of ``scale * q.k`` in fp32 (``fastgen/forward.py:176-258``)."""
+    softmax of ``scale * q.k`` in fp32 (``fastgen/forward.py:176-258``).  With ``sinks`` head ``h``'s softmax runs
+    over one more score, ``sinks[h]`` as it is, whose weight meets no value."""
     n_kv, P, hd = k_pages.shape[1], k_pages.shape[2], k_pages.shape[3]
     G = n_heads // n_kv
     for t in range(q.shape[0]):
@@ -178,7 +225,10 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
         qt = q[t, : n_heads * hd].float().view(n_heads, hd)
         for h in range(n_heads):
             s = (k[lo:, h // G] @ qt[h]) * scale
-            out[t, h * hd : (h + 1) * hd] = (torch.softmax(s, 0) @ v[lo:, h // G]).to(out.dtype)
+            if sinks is not None:
+                s = torch.cat([s, sinks[h].float().reshape(1)])
+            w = torch.softmax(s, 0)[: p + 1 - lo]
+            out[t, h * hd : (h + 1) * hd] = (w @ v[lo:, h // G]).to(out.dtype)
     return out
 
 
@@ -186,7 +236,8 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
                          plan=None, max_chunks=None, min_tiles: int = 4, max_rows: int = 16,
-                         tile_rows=None, exact_weights: bool = False) -> torch.Tensor:
+                         tile_rows=None, exact_weights: bool = False,
+                         sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same attention for tokens listed as items (sequence, first flat token, tokens, position of the
     first token).  How the kernels cut the work (``plan`` and what follows it) does not change the result;
     ``exact_weights`` only says how many digits of the softmax weights the kernel keeps (here: all)."""
@@ -199,16 +250,16 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
             seq_of_token[first : first + n] = b
             positions[first : first + n] = torch.arange(pos, pos + n, dtype=torch.int32)
     return paged_attention_general(q, out, k_pages, v_pages, block_table, seq_of_token, positions, n_heads, scale,
-                                   window)
+                                   window, sinks)
 
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                     group, ctx, n_heads: int, scale: float, window: int = 0,
-                    exact_weights: bool = False) -> torch.Tensor:
+                    exact_weights: bool = False, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of one step: the block table from the layer's cache group, sequences and positions of the
     tokens from the step's context."""
     return paged_attention_general(q, out, k_pages, v_pages, group.block_table, ctx.seq_of_token, ctx.positions,
-                                   n_heads, scale, window)
+                                   n_heads, scale, window, sinks)
 
 
 def gemm_nt(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
@@ -259,10 +310,7 @@ def gemm_skinny(x, w, out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue
                             for s in range(k_splits)])
     y = xf @ wf.T
     if silu_mul_epilogue:
-        M, N = y.shape
-        gu = y.view(M, N // 16, 2, 8)
-        g, u = gu[:, :, 0].reshape(M, N // 2), gu[:, :, 1].reshape(M, N // 2)
-        y = g * torch.sigmoid(g) * u
+        y = _gated(y, silu_mul_epilogue)
     return y.to(out_dtype or torch.bfloat16)
 
 
@@ -278,10 +326,7 @@ def gemm_tiled(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None,
                             for s in range(k_splits)])
     y = xf @ wf.T
     if silu_mul_epilogue:
-        M, N = y.shape
-        gu = y.view(M, N // 16, 2, 8)
-        g, u = gu[:, :, 0].reshape(M, N // 2), gu[:, :, 1].reshape(M, N // 2)
-        y = g * torch.sigmoid(g) * u
+        y = _gated(y, silu_mul_epilogue)
     return y.to(out_dtype or torch.bfloat16)
 
 
@@ -408,3 +453,91 @@ def sample_support(logits: torch.Tensor, temperature: float, top_p: float) -> to
 def logprob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
     """``log_softmax(logits)[row, tokens[row]]`` (``fastgen/generate.py:725-730``)."""
     return torch.log_softmax(logits.float(), -1)[torch.arange(logits.shape[0], device=logits.device), tokens.long()]
+
+
+# ------------------------------------------------------------- per-head work
+def heads_prepare(src: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                  n_q: int = 0, q_col: int = 0, q_width: int = 0, q_norm: Optional[torch.Tensor] = None,
+                  q_norm_dims: int = 0, q_out: Optional[torch.Tensor] = None, q_out_width: int = 0,
+                  n_kv: int = 0, k_col: int = 0, k_width: int = 0, k_norm: Optional[torch.Tensor] = None,
+                  k_norm_dims: int = 0, v_col: int = -1, v_width: int = 0,
+                  table: Optional[torch.Tensor] = None, rot_start: int = 0, rotary_dim: int = 0,
+                  rotate_q: bool = True, rotate_k: bool = True, slots: Optional[torch.Tensor] = None,
+                  k_pages: Optional[torch.Tensor] = None, v_pages: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """Bias, a norm over the first dimensions of each head, the rotation of a run of pairs; queries to ``q_out``
+    and keys and values to their pages, every head padded with zeros to its destination's width."""
+    T = src.shape[0]
+    x = src.float() + (bias.float()[None, : src.shape[1]] if bias is not None else 0.0)
+
+    def heads(col, n, width, norm_w, norm_dims, turn):
+        y = x[:, col : col + n * width].reshape(T, n, width).clone()
+        if norm_w is not None:
+            part = y[..., :norm_dims]
+            y[..., :norm_dims] = part * torch.rsqrt((part * part).mean(-1, keepdim=True) + eps) * norm_w.float()[:norm_dims]
+        if table is not None and rotary_dim and turn:
+            run = y[..., rot_start : rot_start + rotary_dim]
+            y[..., rot_start : rot_start + rotary_dim] = _rotate(run, table, rotary_dim)
+        return y
+
+    if n_q:
+        q = heads(q_col, n_q, q_width, q_norm, q_norm_dims, rotate_q)
+        wide = torch.zeros(T, n_q, q_out_width)
+        wide[..., :q_width] = q.to(q_out.dtype).float().cpu()
+        q_out[:, : n_q * q_out_width] = wide.reshape(T, -1).to(q_out.dtype).to(q_out.device)
+    if n_kv:
+        hd = k_pages.shape[3]
+        k = heads(k_col, n_kv, k_width, k_norm, k_norm_dims, rotate_k)
+        v = k[..., :v_width] if v_col < 0 else x[:, v_col : v_col + n_kv * v_width].reshape(T, n_kv, v_width)
+        kw, vw = torch.zeros(T, n_kv, hd), torch.zeros(T, n_kv, hd)
+        kw[..., :k_width], vw[..., :v_width] = k.cpu(), v.cpu()
+        _write_pages(k_pages, v_pages, slots, kw, vw)
+    return q_out
+
+
+def head_linear(x: torch.Tensor, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_head_stride: int,
+                tail: int = 0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t, h, :N] = w[h] @ x[t, h, :K]`` (times ``sigmoid(gate[t, h])``), then ``tail`` columns of ``x`` copied
+    through, then zeros up to ``out_head_stride``."""
+    H, N, K = w.shape
+    T = x.shape[0]
+    for h in range(H):
+        xh = x[:, h * x_head_stride : h * x_head_stride + K + tail].float()
+        y = xh[:, :K] @ w[h].float().T
+        if gate is not None:
+            y = y * torch.sigmoid(gate[:, h].float())[:, None]
+        full = torch.zeros(T, out_head_stride, device=x.device)
+        full[:, :N] = y
+        full[:, N : N + tail] = xh[:, K:]
+        out[:, h * out_head_stride : (h + 1) * out_head_stride] = full.to(out.dtype)
+    return out
+
+
+def head_norm_gate(x: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor, n_heads: int,
+                   out: torch.Tensor) -> torch.Tensor:
+    """RMS norm of every head of fp32 ``x [T, H*e]`` with one weight ``[e]``, times ``silu(gate)``."""
+    T, e = x.shape[0], x.shape[1] // n_heads
+    y = x.view(T, n_heads, e)
+    y = y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float()
+    g = gate[:, : n_heads * e].float().reshape(T, n_heads, e)
+    out.copy_((y * g * torch.sigmoid(g)).reshape(T, -1).to(out.dtype))
+    return out
+
+
+def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: Optional[torch.Tensor],
+               tau: float, q_scale: float, state: torch.Tensor, slot_ids: torch.Tensor, q_start: torch.Tensor,
+               n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+    """Per sequence and head, token by token: ``S = a[:, None] * S + k v^T``, ``o = S^T (q * q_scale)`` with
+    ``a = sigmoid(z + z_bias) ** (1 / tau)``; ``S`` is the sequence's row of ``state``, updated in place."""
+    _, H, d, e = state.shape
+    for b in range(n_seqs):
+        S = state[int(slot_ids[b])]
+        for t in range(int(q_start[b]), int(q_start[b + 1])):
+            row = qkv[t].float()
+            q = row[q_col : q_col + H * d].view(H, d) * q_scale
+            k = row[k_col : k_col + H * d].view(H, d)
+            v = row[v_col : v_col + H * e].view(H, e)
+            zt = z[t, : H * d].float() + (z_bias.float() if z_bias is not None else 0.0)
+            a = torch.exp(torch.nn.functional.logsigmoid(zt) / tau).view(H, d)
+            S.copy_(a[:, :, None] * S + k[:, :, None] * v[:, None, :])
+            out[t] = torch.einsum("hde,hd->he", S, q).reshape(-1)
+    return out

@@ -63,9 +63,9 @@ class Attention(Mixer):
         self.cache_window: Optional[int] = o.get("cache_window", self.window) or None
         # the width of a head in the cache: keys and values of different widths are padded with zeros to one
         # width, a multiple of 16 (what the matrix-core kernels take)
-        self.cache_dim = self.head_dim if self.v_head_dim == self.head_dim else -(-max(self.head_dim, self.v_head_dim) // 16) * 16
         # the general form: what the product gives goes through a kernel of its own on its way to the attention
-        self.prepared = self.bias or self.qk_norm or not self.has_kv or self.cache_dim != self.head_dim
+        self.prepared = self.bias or self.qk_norm or not self.has_kv or self.v_head_dim != self.head_dim
+        self.cache_dim = -(-max(self.head_dim, self.v_head_dim) // 16) * 16 if self.prepared else self.head_dim
         if self.prepared and (self.value_from_key or self.output_gate):
             raise ValueError(f"{self.prefix}: value_from_key and output_gate do not go with bias, qk_norm, v_head_dim or has_kv")
         if self.v_head_dim % 2 or self.cache_dim > 512:
