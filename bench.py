@@ -6,6 +6,7 @@
     python bench.py --workload readme       # the load of the reference's README, see readme_workload()
     python bench.py --workload readme --shape 70b   # the same load at the 70B sizes, cache = the memory left
     python bench.py --workload buderax      # the Buderax design beside the dense Llama at equal sizes
+    python bench.py --workload gisodra      # the Gisodra design beside the dense Llama at equal sizes
 
 The model has the layer sizes of Llama 3.1 8B (32 layers, hidden 4096, 32
 heads, 8 kv heads, head size 128, feed-forward 14336, vocabulary 128256,
@@ -309,6 +310,163 @@ def buderax_workload(prefill_tokens: int = 2048, batch: int = 8, context: int = 
     return 0
 
 
+# Gisodra at sizes that resemble a real model's layers: eight layers in the order attention, gated linear
+# attention, attention on the first one's cache, latent attention, twice; the dense Llama beside it has the same
+# width, heads, head size, feed-forward width and number of layers.
+GISODRA_SIZES = {
+    "w1024": dict(width=1024, heads=16, kv_heads=4, dim=64, ff=2816, window=1024, gla_heads=8, gla_dim=64, gla_vdim=128,
+                  lat_dim=64, rot_dim=32, kv_rank=192, q_rank=384, vocab=32000),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=5632, window=4096, gla_heads=16, gla_dim=128, gla_vdim=128,
+                  lat_dim=128, rot_dim=64, kv_rank=192, q_rank=768, vocab=32000),
+}
+
+
+def _gisodra_configs(z: dict):
+    attn = lambda **more: dict(type="attention", mlp=dict(kind="dense", ff=z["ff"]), mixer=dict(
+        heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5,
+        mask=dict(size=z["window"]), **more))
+    gla = dict(type="gla", mlp=None, mixer=dict(heads=z["gla_heads"], dim=z["gla_dim"], vdim=z["gla_vdim"], tau=16.0))
+    latent = dict(type="latent_attention", mlp=dict(kind="dense", ff=z["ff"]), mixer=dict(
+        heads=z["heads"], dim=z["lat_dim"], rot_dim=z["rot_dim"], vdim=z["dim"], kv_rank=z["kv_rank"], q_rank=z["q_rank"],
+        scale=(z["lat_dim"] + z["rot_dim"]) ** -0.5, mask=dict(size=z["window"]), rot=dict(base=1000000.0, dims=z["rot_dim"])))
+    layers = [attn(), gla, attn(kv_from=0), latent, attn(), gla, attn(kv_from=4), latent]
+    new = dict(architecture="Gisodra", width=z["width"], vocab=z["vocab"], norm=dict(eps=1e-6), logit_softcap=30.0, layers=layers)
+    dense = dict(architectures=["LlamaForCausalLM"], hidden_size=z["width"], intermediate_size=z["ff"],
+                 num_hidden_layers=len(layers), num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"],
+                 rms_norm_eps=1e-6, vocab_size=z["vocab"], rope_theta=500000.0, rope_scaling=None,
+                 tie_word_embeddings=True, max_position_embeddings=131072)
+    return new, dense
+
+
+def _gisodra_kernels(z: dict, rows: int, context: int) -> dict:
+    """The design's own kernels at ``rows`` tokens (one prompt of ``rows`` tokens, or ``rows`` sequences of one
+    token at ``context`` cached ones), each beside the like kernel of the dense decoder on operands of the same
+    size: microseconds, and the shares of the memory roofline (the bytes the kernel has to move) and of the
+    matrix cores' (its products' flops)."""
+    import torch
+
+    from fastgen_amd.kernels import ops
+    from fastgen_amd.kernels.linear import linear
+
+    D, H, G, d, P = z["width"], z["heads"], z["kv_heads"], z["dim"], PAGE
+    R, r, dl, Q = z["kv_rank"], z["rot_dim"], z["lat_dim"], z["q_rank"]
+    gh, gd, ge = z["gla_heads"], z["gla_dim"], z["gla_vdim"]
+    g = torch.Generator(device="cuda").manual_seed(rows)
+    rnd = lambda *shape: (torch.randn(*shape, generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+    f32 = lambda *shape: torch.randn(*shape, generator=g, device="cuda")
+    decode = rows <= 16
+    n_seqs = rows if decode else 1
+    n_pages = rows // P + 2
+    slots = torch.arange(rows, dtype=torch.int32, device="cuda")
+    table = ops.rope_table(torch.arange(rows, dtype=torch.int32, device="cuda"), f32(max(d, r) // 2).abs())
+    out = {}
+
+    def put(name, fn, nbytes, flops=0):
+        t = _time(fn)
+        out[name] = {"us": round(t * 1e6, 1), "hbm_frac": round(nbytes / t / PEAK_HBM, 4),
+                     "mfma_frac": round(flops / t / PEAK_FLOPS["bf16"], 4)}
+
+    # between the q/k/v product and the attention: bias, norms per head, cache write; beside rotation and cache write
+    qkv32, qkv16 = f32(rows, (H + 2 * G) * d), rnd(rows, (H + 2 * G) * d)
+    bias, nw = f32((H + 2 * G) * d), f32(d)
+    kp, vp = rnd(n_pages, G, P, d), rnd(n_pages, G, d, P)
+    q_out = torch.empty(rows, H * d, dtype=torch.bfloat16, device="cuda")
+    put("heads_prepare (attention)", lambda: ops.heads_prepare(
+        qkv32, bias, 1e-6, n_q=H, q_col=0, q_width=d, q_norm=nw, q_norm_dims=d, q_out=q_out, q_out_width=d, n_kv=G,
+        k_col=H * d, k_width=d, k_norm=nw, k_norm_dims=d, v_col=(H + G) * d, v_width=d, slots=slots, k_pages=kp, v_pages=vp),
+        qkv32.numel() * 4 + (H + 2 * G) * d * rows * 2)
+    table_d = table[:, : d // 2].contiguous()
+    put("rope_kv_write (llama)", lambda: ops.rope_kv_write(qkv16, slots, None, slots, kp, vp, H, G, d, d, table=table_d),
+        qkv16.numel() * 2 + (H + 2 * G) * d * rows * 2)
+    # the norms around a sublayer; beside the one norm of the dense decoder
+    h, delta, w1, w2 = f32(rows, D), rnd(rows, D), rnd(D), rnd(D)
+    normed = torch.empty(rows, D, dtype=torch.bfloat16, device="cuda")
+    put("post_add_rmsnorm", lambda: ops.post_add_rmsnorm(h, delta, w1, 1e-6, w2, 1e-6, normed), rows * D * (4 + 4 + 2 + 2))
+    put("add_rmsnorm (llama)", lambda: ops.add_rmsnorm(h, delta, w2, 1e-6, normed), rows * D * (4 + 4 + 2 + 2))
+    # the feed-forward's first product with its activation
+    x, wgu = rnd(rows, D) * 20, ops.interleave_gate_up(rnd(z["ff"], D), rnd(z["ff"], D))
+    put("gate/up + gelu_tanh", lambda: linear(x, wgu, epilogue="gelu_tanh_mul"), wgu.numel() * 2, 2 * rows * wgu.numel())
+    put("gate/up + silu (llama)", lambda: linear(x, wgu, epilogue="silu_mul"), wgu.numel() * 2, 2 * rows * wgu.numel())
+    # latent attention: the products per head beside one product of the same flops and weights
+    hc = -(-(R + r) // 16) * 16
+    q, w_uk_t = rnd(rows, H * (dl + r)), rnd(H, R, dl)
+    q_lat = torch.empty(rows, H * hc, dtype=torch.bfloat16, device="cuda")
+    put("head_linear (queries into the latent)", lambda: ops.head_linear(q, dl + r, w_uk_t, q_lat, hc, tail=r),
+        w_uk_t.numel() * 2 + q.numel() * 2 + q_lat.numel() * 2, 2 * rows * H * R * dl)
+    lat, w_uv, gate = rnd(rows, H * hc), rnd(H, d, R), f32(rows, H)
+    v_out = torch.empty(rows, H * d, dtype=torch.bfloat16, device="cuda")
+    put("head_linear (outputs out of the latent)", lambda: ops.head_linear(lat, hc, w_uv, v_out, d, gate=gate),
+        w_uv.numel() * 2 + lat.numel() * 2 + v_out.numel() * 2, 2 * rows * H * R * d)
+    xs, wl = rnd(rows, dl), rnd(H * R, dl)
+    put("one product of the same flops (library or own)", lambda: linear(xs, wl), wl.numel() * 2 + rows * (dl + H * R) * 2,
+        2 * rows * H * R * dl)
+    rows32 = f32(rows, Q + R + r + H)
+    cq = torch.empty(rows, Q, dtype=torch.bfloat16, device="cuda")
+    kl, vl = rnd(n_pages, 1, P, hc), rnd(n_pages, 1, hc, P)
+    nq, nk, table_r = f32(Q), f32(R), table[:, : r // 2].contiguous()
+    put("heads_prepare (latents)", lambda: ops.heads_prepare(
+        rows32, None, 1e-6, n_q=1, q_col=0, q_width=Q, q_norm=nq, q_norm_dims=Q, q_out=cq, q_out_width=Q, n_kv=1, k_col=Q,
+        k_width=R + r, k_norm=nk, k_norm_dims=R, v_col=-1, v_width=R, table=table_r, rot_start=R,
+        rotary_dim=r, rotate_q=False, slots=slots, k_pages=kl, v_pages=vl), rows * ((Q + R + r) * 4 + Q * 2 + 2 * hc * 2))
+    # the recurrence: fp32 vector arithmetic, token by token; four flops a state element and token
+    width = 2 * gh * gd + 2 * gh * ge
+    rows16, zz, zb = rnd(rows, width), f32(rows, gh * gd), f32(gh * gd)
+    state = torch.zeros(n_seqs + 1, gh, gd, ge, device="cuda")
+    slot_ids = torch.arange(n_seqs, dtype=torch.int32, device="cuda")
+    q_start = torch.arange(0, rows + 1, rows // n_seqs, dtype=torch.int32, device="cuda")
+    o32 = torch.empty(rows, gh * ge, device="cuda")
+    t = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, state, slot_ids, q_start, n_seqs, o32))
+    out["decay_scan"] = {"us": round(t * 1e6, 1),
+                         "hbm_frac": round((2 * n_seqs * gh * gd * ge * 4 + rows * (width * 2 + gh * gd * 4 + gh * ge * 4)) / t / PEAK_HBM, 4),
+                         "fp32_vector_frac": round(4 * rows * gh * gd * ge / t / 157e12, 4)}
+    gated = torch.empty(rows, gh * ge, dtype=torch.bfloat16, device="cuda")
+    ng = f32(ge)
+    put("head_norm_gate", lambda: ops.head_norm_gate(o32, ng, 1e-6, rows16[:, 2 * gh * gd + gh * ge:], gh, gated),
+        rows * gh * ge * (4 + 2 + 2))
+    return out
+
+
+def gisodra_workload(prefill_tokens: int = 2048, batch: int = 8, context: int = 1024, steps: int = 32, warmup: int = 8) -> int:
+    """Prefill and decode throughput of Gisodra models with random bfloat16 weights beside dense Llama models
+    of equal sizes, and the design's own kernels beside the dense decoder's like ones.  One JSON line."""
+    import torch
+
+    from fastgen_amd.engine import Engine
+
+    results = {}
+    for name, z in GISODRA_SIZES.items():
+        new, dense = _gisodra_configs(z)
+        row = {"layers": len(new["layers"])}
+        for label, cfg in (("gisodra", new), ("llama", dense)):
+            engine = Engine.from_config(cfg, seed=5, dtype=torch.bfloat16, page_size=PAGE,
+                                        max_tokens=max(batch * (context + 256), prefill_tokens + PAGE), max_batch=batch,
+                                        max_step_tokens=prefill_tokens)
+            g = torch.Generator().manual_seed(0)
+            prompt = lambda n: torch.randint(0, z["vocab"], (n,), generator=g).tolist()
+            pre = min(engine.time_prefill(prompt(prefill_tokens), repeats=5))
+            dt = engine.time_decode([prompt(context) for _ in range(batch)], steps=steps, warmup=warmup)
+            row[label] = {"prefill_tok_s": round(prefill_tokens / pre, 1), "prefill_ms": round(pre * 1e3, 3),
+                          "decode_tok_s": round(batch * steps / dt, 1), "decode_ms_per_step": round(dt / steps * 1e3, 4),
+                          "weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
+            print(f"[bench] {name} {label}: {row[label]}", file=sys.stderr, flush=True)
+            del engine
+            torch.cuda.empty_cache()
+        row["kernels_prefill"] = _gisodra_kernels(z, prefill_tokens, context)
+        row["kernels_decode"] = _gisodra_kernels(z, batch, context)
+        print(f"[bench] {name} kernels: {row['kernels_prefill']} {row['kernels_decode']}", file=sys.stderr, flush=True)
+        results[name] = row
+    first = results[next(iter(results))]
+    print(json.dumps({
+        "metric": "Gisodra beside the dense Llama at equal sizes: prefill and decode tok/s", "unit": "tokens/s",
+        "value": first["gisodra"]["decode_tok_s"], "n_gpus": 1, "steps": steps, "warmup": warmup, "higher_is_better": True,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"prefill_tokens": prefill_tokens, "decode_batch": batch, "decode_context": context, "page_size": PAGE,
+                   "sizes": GISODRA_SIZES},
+        "results": results,
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -326,9 +484,9 @@ def main() -> int:
                          " 2,048); more are fed untimed, in portions")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
-    ap.add_argument("--workload", choices=["decode", "serve", "readme", "buderax"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "serve", "readme", "buderax", "gisodra"], default="decode",
                     help="decode (default): the step benchmark; serve: continuous batching of 256 requests; "
-                         "readme: the load of the reference's README; buderax: the Buderax design beside the dense "
+                         "readme: the load of the reference's README; buderax, gisodra: that design beside the dense "
                          "Llama at equal sizes")
     ap.add_argument("--step-budget", type=int, default=2048, help="tokens a step of the serve workload")
     ap.add_argument("--show-choices", action="store_true",
@@ -341,6 +499,8 @@ def main() -> int:
         return serve_workload(step_budget=a.step_budget, shape=a.shape or "3b")
     if a.workload == "readme":
         return readme_workload(a.shape or "8b")
+    if a.workload == "gisodra":
+        return gisodra_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
     if a.workload == "buderax":
         return buderax_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
     a.shape = a.shape or "8b"

@@ -1,6 +1,6 @@
 // A linear recurrence with a decay per key channel (gated linear attention), token by token:
 //
-//   a_t = sigmoid(z_t + b)^(1/tau)                       (per head and key channel, fp32)
+//   a_t = sigmoid(z_t + b)^(1/tau)                       (per head and key channel, fp32; all tokens at once)
 //   S_t = diag(a_t) S_(t-1) + k_t v_t^T                  (per head, [d, e] fp32, kept per request)
 //   o_t = S_t^T (q_t * q_scale)
 //
@@ -9,35 +9,48 @@
 // step holds besides it: the tokens of a sequence are taken in order, each output element is one
 // fixed chain of additions, so a prompt cut into portions or batched with others gives the same bits.
 //
-// grid (B sequences, H heads, ceil(e / 16)); one wave.  Lane l owns value channel 16 z + (l & 15) and
-// the key channels rg * rpl .. rg * rpl + rpl - 1 with rg = l >> 4, rpl = ceil(d / 4): a quarter of a
-// column of S in registers.  q, k and the decays of a few tokens go through LDS.
+// grid (B sequences, H heads, ceil(e / 8)); one wave.  Lane l owns value channel 8 z + (l & 7) and the
+// key channels rg * rpl .. rg * rpl + rpl - 1 with rg = l >> 3, rpl = ceil(d / 8): an eighth of a column
+// of S in registers.  q, k and the decays of a run of tokens go through LDS.
 #include "common.h"
 
-#define RC_TOKENS 4  // tokens staged at a time
+// tokens staged at a time: as many as leave the kernel's registers unspilled
+#define RC_TOKENS_FOR(RPL) ((RPL) <= 8 ? 16 : 8)
 
 struct ScanArgs {
   const void* qkv; int row_stride, q_col, k_col, v_col;  // act dtype rows: q, k [H * d], v [H * e] at their columns
-  const float* z; int z_stride;                          // fp32 [T, >= H * d]: the decay's logits before the bias
-  const float* z_bias;                                   // fp32 [H * d] or null
-  float inv_tau, q_scale;
+  const float* decay; int decay_stride;                  // fp32 [T, >= H * d]: a_t (fg_decay_from_logits)
+  float q_scale;
   float* state;                                          // fp32 [n_slots, H, d, e]
   const int* slot_ids; const int* q_start;               // [B], [B + 1]
   float* out;                                            // fp32 [T, H * e]
   int H, d, e;
 };
 
+// The loop over a sequence's tokens is a chain: what it costs is how many instructions one link takes
+// (a wave issues one every few clocks) and what it waits for.  So the loads of a run of RC_TOKENS tokens
+// (8 or 16; decays, k, q: d of each a token, spread over the lanes; and each lane's own value channel) are all
+// issued into registers before the run before it is computed, and reach LDS (q scaled) when that is
+// done: memory latency passes behind the arithmetic.  The decays come ready from a kernel of their own
+// (exponentials and logarithms of every token at once, not in this chain).  RPL >= ceil(d / 8); NJ =
+// ceil(d / 64) is the number of staged elements a lane holds of each of the three, per token.
 template <class TA, int RPL>
 __global__ __launch_bounds__(FG_WAVE) void decay_scan_kernel(const ScanArgs a) {
-  extern __shared__ float lds[];  // [RC_TOKENS][3][d]: decay, k, q
+  constexpr int NJ = RPL >= 8 ? RPL / 8 : 1;
+  constexpr int RC_TOKENS = RC_TOKENS_FOR(RPL);
+  // [RC_TOKENS][3][d + 32]: decay, k, q; key channel r lies at r + 4 (r / rpl), so that the eight parts
+  // that the lane groups read at once start in different banks and every part is 16-byte aligned
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int lane = threadIdx.x;
   const int b = blockIdx.x, h = blockIdx.y;
-  const int c = lane & 15, rg = lane >> 4;
-  const int col = blockIdx.z * 16 + c;
+  const int c = lane & 7, rg = lane >> 3;
+  const int col = blockIdx.z * 8 + c;
   const bool col_ok = col < a.e;
   const int d = a.d, e = a.e;
-  const int rpl = (d + 3) / 4;
+  const int rpl = (d + 7) / 8;
   const int r0 = rg * rpl;
+  const int ds = d + 32;              // a staged vector's stride
+  const bool vec = rpl % 4 == 0 && d == 8 * rpl;  // uniform: the parts are read as float4
   const int t_begin = a.q_start[b], t_end = a.q_start[b + 1];
   float* S_mem = a.state + (((size_t)a.slot_ids[b] * a.H + h) * d) * e;
   float S[RPL];
@@ -46,42 +59,112 @@ __global__ __launch_bounds__(FG_WAVE) void decay_scan_kernel(const ScanArgs a) {
     const int r = r0 + i;
     S[i] = (i < rpl && r < d && col_ok) ? S_mem[(size_t)r * e + col] : 0.f;
   }
+  const TA* qkv = (const TA*)a.qkv;
+  // the key channels this lane stages (the same for every token): where they come from and where they go
+  int src[NJ], dst[NJ];
+  bool mine[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int r = lane + FG_WAVE * j;
+    mine[j] = r < d;
+    src[j] = h * d + min(r, d - 1);
+    dst[j] = r + 4 * (r / rpl);
+  }
+  const int v_src = a.v_col + h * e + min(col, e - 1);
+  float pa[RC_TOKENS][NJ], pk[RC_TOKENS][NJ], pq[RC_TOKENS][NJ], pv[RC_TOKENS];
+  auto fetch = [&](int t0) {  // the run t0 .. t0 + n - 1 into registers: nothing waits here
+    const int n = min(RC_TOKENS, t_end - t0);
+#pragma unroll
+    for (int tt = 0; tt < RC_TOKENS; ++tt) {
+      const size_t t = (size_t)(t0 + min(tt, n - 1));  // (never conditional: beyond the run, its last token again)
+      const TA* row = qkv + t * a.row_stride;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        pa[tt][j] = a.decay[t * a.decay_stride + src[j]];
+        pk[tt][j] = to_f<TA>(row[a.k_col + src[j]]);
+        pq[tt][j] = to_f<TA>(row[a.q_col + src[j]]);
+      }
+      pv[tt] = to_f<TA>(row[v_src]);
+    }
+  };
+  if (t_begin < t_end) fetch(t_begin);
   for (int t0 = t_begin; t0 < t_end; t0 += RC_TOKENS) {
     const int n = min(RC_TOKENS, t_end - t0);
-    __syncthreads();
-    for (int idx = lane; idx < n * d; idx += FG_WAVE) {
-      const int tt = idx / d, r = idx % d;
-      const size_t t = (size_t)(t0 + tt);
-      float zv = a.z[t * a.z_stride + h * d + r];
-      if (a.z_bias) zv += a.z_bias[h * d + r];
-      // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|)), then the power as a product in the exponent
-      const float ls = fminf(zv, 0.f) - log1pf(expf(-fabsf(zv)));
-      const TA* row = (const TA*)a.qkv + t * a.row_stride;
-      float* dst = lds + (size_t)tt * 3 * d;
-      dst[r] = expf(ls * a.inv_tau);
-      dst[d + r] = to_f<TA>(row[a.k_col + h * d + r]);
-      dst[2 * d + r] = to_f<TA>(row[a.q_col + h * d + r]) * a.q_scale;
-    }
-    __syncthreads();
-    for (int tt = 0; tt < n; ++tt) {
-      const size_t t = (size_t)(t0 + tt);
-      const float* av = lds + (size_t)tt * 3 * d;
-      const float* kv = av + d;
-      const float* qv = kv + d;
-      const float v = col_ok ? to_f<TA>(((const TA*)a.qkv)[t * a.row_stride + a.v_col + h * e + col]) : 0.f;
-      float acc = 0.f;
+    __syncthreads();  // the run before has been read
+    float v[RC_TOKENS];
 #pragma unroll
-      for (int i = 0; i < RPL; ++i) {
-        const int r = r0 + i;
-        if (i < rpl && r < d) {
-          S[i] = av[r] * S[i] + kv[r] * v;
-          acc += S[i] * qv[r];
+    for (int tt = 0; tt < RC_TOKENS; ++tt) {
+      v[tt] = pv[tt];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        if (mine[j]) {
+          float* to = lds + (size_t)tt * 3 * ds + dst[j];
+          to[0] = pa[tt][j];
+          to[ds] = pk[tt][j];
+          to[2 * ds] = pq[tt][j] * a.q_scale;
         }
       }
-      // the four quarters of the column, in a fixed order
-      const float a1 = __shfl(acc, c + 16, FG_WAVE), a2 = __shfl(acc, c + 32, FG_WAVE), a3 = __shfl(acc, c + 48, FG_WAVE);
-      const float a0 = __shfl(acc, c, FG_WAVE);
-      if (rg == 0 && col_ok) a.out[t * ((size_t)a.H * e) + h * e + col] = ((a0 + a1) + a2) + a3;
+    }
+    __syncthreads();
+    if (t0 + RC_TOKENS < t_end) fetch(t0 + RC_TOKENS);  // in flight while this run is computed
+    // One token after the other; the sums over the lane groups are taken for the whole run at once (the
+    // lanes' exchange is the longest link of the chain: sixteen of them wait together).  Reading a token's
+    // operands from LDS a token ahead into a second set of registers was measured slower (the registers spill).
+    float acc[RC_TOKENS];
+    const float* part0 = lds + r0 + 4 * rg;  // this lane group's part of a staged vector
+    if (vec) {
+#pragma unroll
+      for (int tt = 0; tt < RC_TOKENS; ++tt) {
+        const float* av = part0 + (size_t)tt * 3 * ds;
+        // four sums side by side (channels u, u + 4, ..), added up at the end: no chain of dependent additions
+        float part[4] = {0.f, 0.f, 0.f, 0.f};
+        if (tt < n) {
+#pragma unroll
+          for (int i4 = 0; i4 < RPL / 4; ++i4) {
+            if (4 * i4 < rpl) {
+              const float4 a4 = ((const float4*)av)[i4], k4 = ((const float4*)(av + ds))[i4],
+                           q4 = ((const float4*)(av + 2 * ds))[i4];
+              const float aa[4] = {a4.x, a4.y, a4.z, a4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, qq[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+              for (int u = 0; u < 4; ++u) {
+                S[4 * i4 + u] = aa[u] * S[4 * i4 + u] + kk[u] * v[tt];
+                part[u] += S[4 * i4 + u] * qq[u];
+              }
+            }
+          }
+        }
+        acc[tt] = (part[0] + part[1]) + (part[2] + part[3]);
+      }
+    } else {
+#pragma unroll
+      for (int tt = 0; tt < RC_TOKENS; ++tt) {
+        const float* av = part0 + (size_t)tt * 3 * ds;
+        float sum = 0.f;
+        if (tt < n) {
+#pragma unroll
+          for (int i = 0; i < RPL; ++i) {
+            if (i < rpl && r0 + i < d) {
+              S[i] = av[i] * S[i] + av[ds + i] * v[tt];
+              sum += S[i] * av[2 * ds + i];
+            }
+          }
+        }
+        acc[tt] = sum;
+      }
+    }
+    // the eight parts of a column: a butterfly whose order of additions is the same in every lane
+#pragma unroll
+    for (int m = 8; m < FG_WAVE; m <<= 1) {
+      float other[RC_TOKENS];
+#pragma unroll
+      for (int tt = 0; tt < RC_TOKENS; ++tt) other[tt] = __shfl_xor(acc[tt], m, FG_WAVE);
+#pragma unroll
+      for (int tt = 0; tt < RC_TOKENS; ++tt) acc[tt] += other[tt];
+    }
+    if (rg == 0 && col_ok) {
+#pragma unroll
+      for (int tt = 0; tt < RC_TOKENS; ++tt)
+        if (tt < n) a.out[(size_t)(t0 + tt) * ((size_t)a.H * e) + h * e + col] = acc[tt];
     }
   }
 #pragma unroll
@@ -91,22 +174,46 @@ __global__ __launch_bounds__(FG_WAVE) void decay_scan_kernel(const ScanArgs a) {
   }
 }
 
+// out[t, c] = sigmoid(z[t, c] + bias[c])^(1/tau) for c < width, as exp(log sigmoid(.) / tau) with
+// log sigmoid(x) = min(x, 0) - log1p(exp(-|x|)); fp32.
+__global__ __launch_bounds__(256) void decay_from_logits_kernel(const float* __restrict__ z, int z_stride,
+                                                                const float* __restrict__ bias, float inv_tau,
+                                                                float* __restrict__ out, int width) {
+  const size_t t = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  const float x = z[t * z_stride + c] + (bias ? bias[c] : 0.f);
+  out[t * width + c] = expf((fminf(x, 0.f) - log1pf(expf(-fabsf(x)))) * inv_tau);
+}
+
+extern "C" int fg_decay_from_logits(const float* z, int z_stride, const float* bias, float inv_tau, float* out,
+                                    int n_rows, int width, hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (width <= 0 || z_stride < width || !(inv_tau > 0.f) || !z || !out) return FG_ERR_ARG;
+  for (int r0 = 0; r0 < n_rows; r0 += 65535) {
+    const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    decay_from_logits_kernel<<<dim3((width + 255) / 256, nr), 256, 0, stream>>>(
+        z + (size_t)r0 * z_stride, z_stride, bias, inv_tau, out + (size_t)r0 * width, width);
+  }
+  return fg_launch_status();
+}
+
 extern "C" int fg_decay_scan(const ScanArgs* args, int n_seqs, int act_dtype, hipStream_t stream) {
   if (n_seqs <= 0) return FG_OK;
   const ScanArgs& a = *args;
-  if (a.H <= 0 || a.d <= 0 || a.d > 256 || a.e <= 0 || a.H > 65535 || (a.e + 15) / 16 > 65535 || !a.qkv || !a.z ||
-      !a.state || !a.slot_ids || !a.q_start || !a.out || !(a.inv_tau > 0.f))
+  if (a.H <= 0 || a.d <= 0 || a.d > 256 || a.e <= 0 || a.H > 65535 || (a.e + 7) / 8 > 65535 || !a.qkv || !a.decay ||
+      !a.state || !a.slot_ids || !a.q_start || !a.out)
     return FG_ERR_ARG;
-  dim3 grid(n_seqs, a.H, (a.e + 15) / 16);
-  const size_t lds = (size_t)RC_TOKENS * 3 * a.d * sizeof(float);
-  const int rpl = (a.d + 3) / 4;
-#define GO(TA, RPL) decay_scan_kernel<TA, RPL><<<grid, FG_WAVE, lds, stream>>>(a)
+  dim3 grid(n_seqs, a.H, (a.e + 7) / 8);
+  const int rpl = (a.d + 7) / 8;
+#define GO(TA, RPL) \
+  decay_scan_kernel<TA, RPL><<<grid, FG_WAVE, (size_t)RC_TOKENS_FOR(RPL) * 3 * (a.d + 32) * sizeof(float), stream>>>(a)
 #define LAUNCH(TA)               \
   do {                           \
-    if (rpl <= 8) GO(TA, 8);     \
+    if (rpl <= 4) GO(TA, 4);     \
+    else if (rpl <= 8) GO(TA, 8);   \
     else if (rpl <= 16) GO(TA, 16); \
-    else if (rpl <= 32) GO(TA, 32); \
-    else GO(TA, 64);             \
+    else GO(TA, 32);             \
   } while (0)
   if (act_dtype == FG_F32) LAUNCH(float);
   else if (act_dtype == FG_BF16) LAUNCH(bf16_t);

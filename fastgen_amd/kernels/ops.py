@@ -1260,8 +1260,8 @@ def head_norm_gate(x: torch.Tensor, weight: torch.Tensor, eps: float, gate: torc
 # ---------------------------------------------------------------- recurrence
 class _ScanArgs(ctypes.Structure):
     _fields_ = [("qkv", ctypes.c_void_p), ("row_stride", ctypes.c_int), ("q_col", ctypes.c_int), ("k_col", ctypes.c_int),
-                ("v_col", ctypes.c_int), ("z", ctypes.c_void_p), ("z_stride", ctypes.c_int), ("z_bias", ctypes.c_void_p),
-                ("inv_tau", ctypes.c_float), ("q_scale", ctypes.c_float), ("state", ctypes.c_void_p),
+                ("v_col", ctypes.c_int), ("decay", ctypes.c_void_p), ("decay_stride", ctypes.c_int),
+                ("q_scale", ctypes.c_float), ("state", ctypes.c_void_p),
                 ("slot_ids", ctypes.c_void_p), ("q_start", ctypes.c_void_p), ("out", ctypes.c_void_p),
                 ("H", ctypes.c_int), ("d", ctypes.c_int), ("e", ctypes.c_int)]
 
@@ -1291,9 +1291,14 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
     _need(d <= 256 and tau > 0, "at most 256 key channels a head; tau positive")
     a = _ScanArgs()
     a.qkv, a.row_stride, a.q_col, a.k_col, a.v_col = qkv.data_ptr(), qkv.stride(0), q_col, k_col, v_col
-    a.z, a.z_stride, a.z_bias = z.data_ptr(), z.stride(0), z_bias.data_ptr() if z_bias is not None else None
-    a.inv_tau, a.q_scale, a.state = 1.0 / tau, q_scale, state.data_ptr()
+    # the decays of every token at once (exponentials and logarithms stay out of the chain of tokens)
+    lib = _lib.load("recurrence")
+    decay = torch.empty((T, H * d), dtype=torch.float32, device=z.device)
+    st = lib.fg_decay_from_logits(_ptr(z), z.stride(0), _ptr(z_bias), ctypes.c_float(1.0 / tau), _ptr(decay), T, H * d,
+                                  _stream(z))
+    _check(st, "decay_from_logits")
+    a.decay, a.decay_stride, a.q_scale, a.state = decay.data_ptr(), decay.stride(0), q_scale, state.data_ptr()
     a.slot_ids, a.q_start, a.out, a.H, a.d, a.e = slot_ids.data_ptr(), q_start.data_ptr(), out.data_ptr(), H, d, e
-    st = _lib.load("recurrence").fg_decay_scan(ctypes.byref(a), int(n_seqs), _code(qkv), _stream(qkv))
+    st = lib.fg_decay_scan(ctypes.byref(a), int(n_seqs), _code(qkv), _stream(qkv))
     _check(st, "decay_scan")
     return out
