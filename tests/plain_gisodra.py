@@ -335,3 +335,15 @@ ONLY_ATTENTION = _config(48, 61, [{"type": "attention", "mixer": _attn(2, 1, 16,
 ONLY_GLA = _config(48, 61, [{"type": "gla", "mixer": {"heads": 2, "dim": 24, "vdim": 8, "tau": 16.0}, "mlp": None}])
 ONLY_LATENT = _config(48, 61, [{"type": "latent_attention", "mixer": _latent(2, 16, 8, 16, 32, 16, 33),
                                 "mlp": None}])
+# sizes that are no multiples of 8 or 16, head counts that are no powers of two, more heads a kv head than the
+# matrix-core kernels take, a window of one token and one longer than any prompt of the tests, a cache read by two
+# later layers through a shorter and a longer window than its owner's, a width that the streaming products refuse
+ODD_SIZES = _config(100, 101, [
+    {"type": "gla", "mixer": {"heads": 3, "dim": 20, "vdim": 12, "tau": 2.5, "decay_rank": 6}, "mlp": {"kind": "dense", "ff": 70}},
+    {"type": "attention", "mixer": _attn(5, 5, 40, 24, 1), "mlp": None},
+    {"type": "latent_attention", "mixer": _latent(7, 20, 6, 10, 30, 18, 1000), "mlp": {"kind": "dense", "ff": 36}},
+    {"type": "attention", "mixer": _attn(34, 2, 8, 8, 50), "mlp": None},
+    {"type": "attention", "mixer": _attn(34, 2, 8, 8, 7, kv_from=3), "mlp": {"kind": "dense", "ff": 24}},
+    {"type": "latent_attention", "mixer": _latent(20, 8, 24, 56, 72, 64, 31, base=77.0), "mlp": None},
+    {"type": "attention", "mixer": _attn(34, 2, 8, 8, 90, kv_from=3), "mlp": None},
+], cap=50.0, eps=1e-4)

@@ -12,12 +12,12 @@ import torch
 from fastgen_amd.config import ConfigError, get_architecture
 from fastgen_amd.engine.model import build_parts
 from fastgen_amd.kernels import twins
-from plain_gisodra import (ONLY_ATTENTION, ONLY_GLA, ONLY_LATENT, TRIO, WIDE_VALUES, plain_decay, plain_decayed_state_scan,
+from plain_gisodra import (ODD_SIZES, ONLY_ATTENTION, ONLY_GLA, ONLY_LATENT, TRIO, WIDE_VALUES, plain_decay, plain_decayed_state_scan,
                            plain_gelu_tanh, plain_gisodra_forward, plain_gisodra_shapes, plain_gisodra_weights,
                            plain_rms, plain_rotate_halves, plain_window_sink_attention)
 
 CONFIGS = {"trio": TRIO, "wide_values": WIDE_VALUES, "only_attention": ONLY_ATTENTION, "only_gla": ONLY_GLA,
-           "only_latent": ONLY_LATENT}
+           "only_latent": ONLY_LATENT, "odd_sizes": ODD_SIZES}
 
 
 # ------------------------------------------------------------------ configuration

@@ -13,13 +13,13 @@ import torch
 
 import traces
 from helpers import assert_close, make_runner, run_trace, save_model_folder
-from plain_gisodra import (ONLY_ATTENTION, ONLY_GLA, ONLY_LATENT, TRIO, WIDE_VALUES, plain_gisodra_forward,
+from plain_gisodra import (ODD_SIZES, ONLY_ATTENTION, ONLY_GLA, ONLY_LATENT, TRIO, WIDE_VALUES, plain_gisodra_forward,
                            plain_gisodra_greedy, plain_gisodra_weights)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 CONFIGS = {"trio": TRIO, "wide_values": WIDE_VALUES, "only_attention": ONLY_ATTENTION, "only_gla": ONLY_GLA,
-           "only_latent": ONLY_LATENT}
+           "only_latent": ONLY_LATENT, "odd_sizes": ODD_SIZES}
 
 
 def _tokens(config, lengths: Dict[str, int], seed: int) -> Dict[str, List[int]]:
