@@ -415,7 +415,13 @@ def _gisodra_kernels(z: dict, rows: int, context: int) -> dict:
     slot_ids = torch.arange(n_seqs, dtype=torch.int32, device="cuda")
     q_start = torch.arange(0, rows + 1, rows // n_seqs, dtype=torch.int32, device="cuda")
     o32 = torch.empty(rows, gh * ge, device="cuda")
-    t = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, state, slot_ids, q_start, n_seqs, o32))
+    q_start_host = q_start.cpu().numpy()  # (with it, long runs of tokens are scanned in chunks side by side)
+    t = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, state, slot_ids, q_start, n_seqs,
+                                     o32, q_start_host=q_start_host))
+    if not decode:
+        t_chain = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, state, slot_ids, q_start,
+                                               n_seqs, o32))
+        out["decay_scan, token by token"] = {"us": round(t_chain * 1e6, 1)}
     out["decay_scan"] = {"us": round(t * 1e6, 1),
                          "hbm_frac": round((2 * n_seqs * gh * gd * ge * 4 + rows * (width * 2 + gh * gd * 4 + gh * ge * 4)) / t / PEAK_HBM, 4),
                          "fp32_vector_frac": round(4 * rows * gh * gd * ge / t / 157e12, 4)}

@@ -25,6 +25,7 @@ struct ScanArgs {
   const int* slot_ids; const int* q_start;               // [B], [B + 1]
   float* out;                                            // fp32 [T, H * e]
   int H, d, e;
+  int write_out, write_state;                            // what a sequence leaves: its tokens' outputs, its last state
 };
 
 // The loop over a sequence's tokens is a chain: what it costs is how many instructions one link takes
@@ -161,7 +162,7 @@ __global__ __launch_bounds__(FG_WAVE) void decay_scan_kernel(const ScanArgs a) {
 #pragma unroll
       for (int tt = 0; tt < RC_TOKENS; ++tt) acc[tt] += other[tt];
     }
-    if (rg == 0 && col_ok) {
+    if (rg == 0 && col_ok && a.write_out) {
 #pragma unroll
       for (int tt = 0; tt < RC_TOKENS; ++tt)
         if (tt < n) a.out[(size_t)(t0 + tt) * ((size_t)a.H * e) + h * e + col] = acc[tt];
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(FG_WAVE) void decay_scan_kernel(const ScanArgs a) {
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
     const int r = r0 + i;
-    if (i < rpl && r < d && col_ok) S_mem[(size_t)r * e + col] = S[i];
+    if (i < rpl && r < d && col_ok && a.write_state) S_mem[(size_t)r * e + col] = S[i];
   }
 }
 
@@ -195,6 +196,66 @@ extern "C" int fg_decay_from_logits(const float* z, int z_stride, const float* b
     decay_from_logits_kernel<<<dim3((width + 255) / 256, nr), 256, 0, stream>>>(
         z + (size_t)r0 * z_stride, z_stride, bias, inv_tau, out + (size_t)r0 * width, width);
   }
+  return fg_launch_status();
+}
+
+// ------------------------------------------------------------ long prompts, chunk by chunk
+// A long run of tokens is cut into chunks that are scanned side by side: first every chunk from a zero
+// state (fg_decay_scan on the chunks as if they were sequences, states only), then, chunk after chunk of a
+// sequence, the state each chunk starts from (below), then every chunk again from its true start, for
+// the outputs.  Twice the arithmetic, as many times the waves as a sequence has chunks.
+//
+// prod[c, j] = the product of decay[t, j] over chunk c's tokens (chunk_start[c] .. chunk_start[c + 1] - 1).
+__global__ __launch_bounds__(256) void decay_chunk_product_kernel(const float* __restrict__ decay, int decay_stride,
+                                                                  const int* __restrict__ chunk_start,
+                                                                  float* __restrict__ prod, int width) {
+  const int c = blockIdx.y, j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= width) return;
+  float p = 1.f;
+  for (int t = chunk_start[c]; t < chunk_start[c + 1]; ++t) p *= decay[(size_t)t * decay_stride + j];
+  prod[(size_t)c * width + j] = p;
+}
+
+// chunks [H, d, e] per chunk holds what each chunk adds to a zero state; it leaves with the state each chunk
+// starts from: for sequence b's chunks c = seq_chunk[b] .. seq_chunk[b + 1] - 1 in order,
+// start(c) = S; S = prod[c] * S + chunks[c], from S = state[slot_ids[b]], which takes the last S.
+__global__ __launch_bounds__(256) void decay_chunk_states_kernel(float* __restrict__ chunks, const float* __restrict__ prod,
+                                                                 float* __restrict__ state, const int* __restrict__ slot_ids,
+                                                                 const int* __restrict__ seq_chunk, int H, int d, int e) {
+  const int b = blockIdx.y;
+  const size_t per = (size_t)H * d * e;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // (head, key channel, value channel)
+  if (i >= per) return;
+  const size_t row = i / e;  // (head, key channel)
+  float* S_mem = state + (size_t)slot_ids[b] * per + i;
+  float S = *S_mem;
+  for (int c = seq_chunk[b]; c < seq_chunk[b + 1]; ++c) {
+    float* at = chunks + (size_t)c * per + i;
+    const float add = *at;
+    *at = S;
+    S = prod[(size_t)c * H * d + row] * S + add;
+  }
+  *S_mem = S;
+}
+
+extern "C" int fg_decay_chunk_product(const float* decay, int decay_stride, const int* chunk_start, float* prod,
+                                      int n_chunks, int width, hipStream_t stream) {
+  if (n_chunks <= 0) return FG_OK;
+  if (width <= 0 || decay_stride < width || n_chunks > 65535 || !decay || !chunk_start || !prod) return FG_ERR_ARG;
+  decay_chunk_product_kernel<<<dim3((width + 255) / 256, n_chunks), 256, 0, stream>>>(decay, decay_stride, chunk_start,
+                                                                                      prod, width);
+  return fg_launch_status();
+}
+
+extern "C" int fg_decay_chunk_states(float* chunks, const float* prod, float* state, const int* slot_ids,
+                                     const int* seq_chunk, int n_seqs, int H, int d, int e, hipStream_t stream) {
+  if (n_seqs <= 0) return FG_OK;
+  const long long per = (long long)H * d * e;
+  if (H <= 0 || d <= 0 || e <= 0 || n_seqs > 65535 || (per + 255) / 256 > 2147483647LL || !chunks || !prod || !state ||
+      !slot_ids || !seq_chunk)
+    return FG_ERR_ARG;
+  decay_chunk_states_kernel<<<dim3((unsigned)((per + 255) / 256), n_seqs), 256, 0, stream>>>(chunks, prod, state, slot_ids,
+                                                                                             seq_chunk, H, d, e);
   return fg_launch_status();
 }
 

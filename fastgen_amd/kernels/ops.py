@@ -1263,19 +1263,29 @@ class _ScanArgs(ctypes.Structure):
                 ("v_col", ctypes.c_int), ("decay", ctypes.c_void_p), ("decay_stride", ctypes.c_int),
                 ("q_scale", ctypes.c_float), ("state", ctypes.c_void_p),
                 ("slot_ids", ctypes.c_void_p), ("q_start", ctypes.c_void_p), ("out", ctypes.c_void_p),
-                ("H", ctypes.c_int), ("d", ctypes.c_int), ("e", ctypes.c_int)]
+                ("H", ctypes.c_int), ("d", ctypes.c_int), ("e", ctypes.c_int), ("write_out", ctypes.c_int),
+                ("write_state", ctypes.c_int)]
+
+
+SCAN_CHUNK = 128  # tokens of a chunk where long runs of tokens are scanned chunk by chunk, side by side
+SCAN_CHUNKED_FROM = 256  # the shortest run of tokens of one sequence for which a step is scanned so
 
 
 def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: Optional[torch.Tensor],
                tau: float, q_scale: float, state: torch.Tensor, slot_ids: torch.Tensor, q_start: torch.Tensor,
-               n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+               n_seqs: int, out: torch.Tensor, q_start_host=None) -> torch.Tensor:
     """The recurrence ``S <- diag(a_t) S + k_t v_t^T``, ``o_t = S^T (q_t * q_scale)`` with
     ``a_t = sigmoid(z_t + z_bias)^(1/tau)``, token by token for every sequence of the step.
 
     ``qkv [T, width]`` holds per token ``q`` and ``k`` (``H*d`` columns from ``q_col`` / ``k_col``) and ``v``
     (``H*e`` from ``v_col``); ``z`` is fp32 ``[T, >= H*d]``; ``state`` fp32 ``[n_slots, H, d, e]`` is read at
     ``slot_ids[b]`` and left as the sequence's last token leaves it; sequence ``b`` has the tokens
-    ``q_start[b] .. q_start[b+1]-1``; ``out`` is fp32 ``[T, H*e]``."""
+    ``q_start[b] .. q_start[b+1]-1``; ``out`` is fp32 ``[T, H*e]``.
+
+    ``q_start_host``: ``q_start`` on the host.  With it, a step in which a sequence brings ``SCAN_CHUNKED_FROM``
+    tokens or more is scanned in chunks of ``SCAN_CHUNK`` tokens side by side (every chunk from a zero state,
+    then the states that the chunks start from, then every chunk from its start); the result differs from
+    the token-by-token scan's by rounding (a chunk's start state is summed in another order)."""
     _gpu(qkv, z, z_bias, state, slot_ids, q_start, out)
     _need(state.dtype == torch.float32 and state.dim() == 4 and state.is_contiguous(), "state must be contiguous float32 [n_slots, H, d, e]")
     _, H, d, e = state.shape
@@ -1299,6 +1309,31 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
     _check(st, "decay_from_logits")
     a.decay, a.decay_stride, a.q_scale, a.state = decay.data_ptr(), decay.stride(0), q_scale, state.data_ptr()
     a.slot_ids, a.q_start, a.out, a.H, a.d, a.e = slot_ids.data_ptr(), q_start.data_ptr(), out.data_ptr(), H, d, e
-    st = lib.fg_decay_scan(ctypes.byref(a), int(n_seqs), _code(qkv), _stream(qkv))
-    _check(st, "decay_scan")
+    a.write_out = a.write_state = 1
+    lens = np.diff(np.asarray(q_start_host[: n_seqs + 1])) if q_start_host is not None else None
+    if lens is None or not len(lens) or int(lens.max()) < SCAN_CHUNKED_FROM or torch.cuda.is_current_stream_capturing():
+        st = lib.fg_decay_scan(ctypes.byref(a), int(n_seqs), _code(qkv), _stream(qkv))
+        _check(st, "decay_scan")
+        return out
+    # chunk by chunk: the chunks' first tokens, and which chunks each sequence has
+    starts, seq_chunk = [], [0]
+    for b in range(n_seqs):
+        starts.extend(range(int(q_start_host[b]), int(q_start_host[b + 1]), SCAN_CHUNK))
+        seq_chunk.append(len(starts))
+    n_chunks = len(starts)
+    _need(n_chunks <= 65535 and n_seqs <= 65535, "too many chunks or sequences in one step")
+    plan = upload(np.asarray(starts + [int(q_start_host[n_seqs])] + seq_chunk + list(range(n_chunks)), dtype=np.int32),
+                  torch.int32, qkv.device)
+    chunk_start, seq_chunk_d, chunk_ids = plan[: n_chunks + 1], plan[n_chunks + 1 : n_chunks + n_seqs + 2], plan[n_chunks + n_seqs + 2 :]
+    chunks = torch.zeros((n_chunks, H, d, e), dtype=torch.float32, device=qkv.device)
+    prod = torch.empty((n_chunks, H * d), dtype=torch.float32, device=qkv.device)
+    _check(lib.fg_decay_chunk_product(_ptr(decay), decay.stride(0), _ptr(chunk_start), _ptr(prod), n_chunks, H * d,
+                                      _stream(qkv)), "decay_chunk_product")
+    a.state, a.slot_ids, a.q_start = chunks.data_ptr(), chunk_ids.data_ptr(), chunk_start.data_ptr()
+    a.write_out, a.write_state = 0, 1  # what every chunk adds to a zero state
+    _check(lib.fg_decay_scan(ctypes.byref(a), n_chunks, _code(qkv), _stream(qkv)), "decay_scan (chunks' sums)")
+    _check(lib.fg_decay_chunk_states(_ptr(chunks), _ptr(prod), _ptr(state), _ptr(slot_ids), _ptr(seq_chunk_d), int(n_seqs),
+                                     H, d, e, _stream(qkv)), "decay_chunk_states")
+    a.write_out, a.write_state = 1, 0  # every chunk from the state it starts from
+    _check(lib.fg_decay_scan(ctypes.byref(a), n_chunks, _code(qkv), _stream(qkv)), "decay_scan (chunks' outputs)")
     return out

@@ -525,9 +525,10 @@ def head_norm_gate(x: torch.Tensor, weight: torch.Tensor, eps: float, gate: torc
 
 def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: Optional[torch.Tensor],
                tau: float, q_scale: float, state: torch.Tensor, slot_ids: torch.Tensor, q_start: torch.Tensor,
-               n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+               n_seqs: int, out: torch.Tensor, q_start_host=None) -> torch.Tensor:
     """Per sequence and head, token by token: ``S = a[:, None] * S + k v^T``, ``o = S^T (q * q_scale)`` with
-    ``a = sigmoid(z + z_bias) ** (1 / tau)``; ``S`` is the sequence's row of ``state``, updated in place."""
+    ``a = sigmoid(z + z_bias) ** (1 / tau)``; ``S`` is the sequence's row of ``state``, updated in place.
+    (``q_start_host`` only lets the kernels cut long runs of tokens into chunks.)"""
     _, H, d, e = state.shape
     for b in range(n_seqs):
         S = state[int(slot_ids[b])]

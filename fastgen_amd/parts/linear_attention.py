@@ -5,7 +5,8 @@ Per head a state ``S [head_dim, v_head_dim]`` in fp32 lives in the request's sta
 per key channel ``a_t = sigmoid(z_t)^(1/tau)``, ``z = W_a2 (W_a1 x) + b`` (a projection through a
 narrow middle).  Each head's output is RMS-normed (one weight for all heads), multiplied by
 ``silu(W_g x)`` and projected.  The recurrence runs token by token in fp32
-(``csrc/recurrence.hip``): what it gives for a token does not depend on how the prompt was cut.
+(``csrc/recurrence.hip``): what it gives for a token does not depend on how the prompt was cut (beyond
+rounding where a step brings hundreds of tokens of a sequence, which are scanned in chunks side by side).
 
 Options: ``dim``, ``n_heads``, ``head_dim``, ``v_head_dim``, ``tau``, ``decay_rank``, ``eps``.
 """
@@ -75,7 +76,7 @@ class GatedLinearAttention(Mixer):
         z = linear(rows[:, a_col : a_col + low], self.w_a2, out_dtype=torch.float32)
         o = torch.empty((T, H * e), dtype=torch.float32, device=x.device)
         ops.decay_scan(rows, 0, k_col, v_col, z, self.a2_bias, self.tau, d ** -0.5, store.state, ctx.slot_ids,
-                       ctx.q_start, ctx.n_seqs, o)
+                       ctx.q_start, ctx.n_seqs, o, q_start_host=None if ctx.graph_capacity else ctx.q_start_host)
         out = torch.empty((T, H * e), dtype=x.dtype, device=x.device)
         ops.head_norm_gate(o, self.norm_w, self.eps, rows[:, g_col:], H, out)
         return linear(out, self.wo, partials_ok=True)

@@ -150,8 +150,10 @@ def test_head_linear_kernel(dtype, T, H, N, K, tail, pad):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,d,e,lens", [(2, 6, 5, [5, 1, 8]), (4, 48, 32, [70, 1, 1, 33]), (1, 256, 24, [9]),
-                                        (3, 20, 130, [2, 40])])
+                                        (3, 20, 130, [2, 40]), (2, 64, 40, [300, 1, 520, 5, 128, 129])])
 def test_decay_scan_and_head_norm_gate_kernels(dtype, H, d, e, lens):
+    """The last case brings runs of hundreds of tokens: with the sequences' starts on the host the kernels scan
+    them in chunks side by side, which must give the token-by-token result within rounding."""
     from fastgen_amd.kernels import ops, twins
 
     g = torch.Generator().manual_seed(d + e)
@@ -168,6 +170,13 @@ def test_decay_scan_and_head_norm_gate_kernels(dtype, H, d, e, lens):
                    q_start.to(DEV), B, og)
     torch.testing.assert_close(og.cpu(), oc, rtol=1e-4, atol=1e-4)
     torch.testing.assert_close(sg.cpu(), sc, rtol=1e-4, atol=1e-4)
+    if max(lens) >= ops.SCAN_CHUNKED_FROM:
+        og2, sg2 = torch.empty(T, H * e, device=DEV), state.to(DEV)
+        ops.decay_scan(rows.to(DEV), 0, H * d, 2 * H * d, z.to(DEV), zb.to(DEV), 4.0, d ** -0.5, sg2, slots.to(DEV),
+                       q_start.to(DEV), B, og2, q_start_host=q_start.numpy())
+        assert not torch.equal(og2, og), "the chunked scan did not run"
+        torch.testing.assert_close(og2.cpu(), oc, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(sg2.cpu(), sc, rtol=1e-4, atol=1e-4)
     wn = torch.rand(e, generator=g) + 0.5
     rc, rg = torch.empty(T, H * e, dtype=dtype), torch.empty(T, H * e, dtype=dtype, device=DEV)
     g_col = 2 * H * d + H * e
@@ -332,6 +341,29 @@ def test_long_decoding_across_pages_and_windows(cases, dtype, name):
     got = run_trace(runner, traces.tail({"z": 200}, 190), toks)
     noise = {"z": plain_gisodra_forward(weights, config, toks["z"], torch.bfloat16)} if dtype == torch.bfloat16 else None
     assert_close(got, want, dtype, noise, f"gisodra {name} long decoding")
+
+
+@pytest.mark.parametrize("name", ["trio", "only_gla", "odd_sizes"])
+def test_long_prompts_whose_recurrence_is_scanned_in_chunks(cases, name):
+    """Prompts of several hundred tokens in one step (the recurrence then runs chunk by chunk, side by side),
+    in two steps and in small portions (token by token): the plain logits, in both precisions, and in float32
+    the cuts agree within rounding."""
+    config, weights, folder, _, _ = cases[name]
+    lengths = {"p": 700, "q": 260, "r": 3}
+    toks = _tokens(config, lengths, seed=13)
+    want = {r: plain_gisodra_forward(weights, config, t) for r, t in toks.items()}
+    exact = {r: plain_gisodra_forward(weights, config, t, torch.float64) for r, t in toks.items()}
+    noise = {r: plain_gisodra_forward(weights, config, t, torch.bfloat16) for r, t in toks.items()}
+    together = [([("p", 0, 700), ("q", 0, 260), ("r", 0, 3)], ["p", "q", "r"])]
+    for dtype in (torch.float32, torch.bfloat16):
+        runner = make_runner(folder, dtype, page_size=16, max_tokens=1024, max_requests=3)
+        for kind, tr in (("whole", traces.whole(lengths)), ("together", together),
+                         ("halves", traces.chunks(lengths, sizes=(390, 310))), ("portions", traces.chunks(lengths))):
+            got = run_trace(runner, tr, toks)
+            if dtype == torch.float32:
+                assert_close(got, exact, dtype, want, f"gisodra {name} long {kind}")
+            else:
+                assert_close(got, want, dtype, noise, f"gisodra {name} long {kind} bfloat16")
 
 
 def test_the_recurrence_remembers_a_far_token(tmp_path):
