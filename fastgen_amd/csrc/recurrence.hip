@@ -7,7 +7,8 @@
 // The state lives in fp32 in a slot per request and is carried from step to step; a step brings a
 // run of tokens per sequence (one when decoding).  Every token's arithmetic is the same whatever the
 // step holds besides it: the tokens of a sequence are taken in order, each output element is one
-// fixed chain of additions, so a prompt cut into portions or batched with others gives the same bits.
+// fixed chain of additions, so a prompt cut into portions or batched with others gives the same bits
+// (long runs of tokens may instead be scanned chunk by chunk, see below: the same within rounding).
 //
 // grid (B sequences, H heads, ceil(e / 8)); one wave.  Lane l owns value channel 8 z + (l & 7) and the
 // key channels rg * rpl .. rg * rpl + rpl - 1 with rg = l >> 3, rpl = ceil(d / 8): an eighth of a column
@@ -15,7 +16,7 @@
 #include "common.h"
 
 // tokens staged at a time: as many as leave the kernel's registers unspilled
-#define RC_TOKENS_FOR(RPL) ((RPL) <= 8 ? 16 : 8)
+#define RC_TOKENS_FOR(RPL) ((RPL) <= 8 ? 16 : (RPL) <= 32 ? 8 : 4)
 
 struct ScanArgs {
   const void* qkv; int row_stride, q_col, k_col, v_col;  // act dtype rows: q, k [H * d], v [H * e] at their columns
@@ -30,7 +31,7 @@ struct ScanArgs {
 
 // The loop over a sequence's tokens is a chain: what it costs is how many instructions one link takes
 // (a wave issues one every few clocks) and what it waits for.  So the loads of a run of RC_TOKENS tokens
-// (8 or 16; decays, k, q: d of each a token, spread over the lanes; and each lane's own value channel) are all
+// (4, 8 or 16; decays, k, q: d of each a token, spread over the lanes; and each lane's own value channel) are all
 // issued into registers before the run before it is computed, and reach LDS (q scaled) when that is
 // done: memory latency passes behind the arithmetic.  The decays come ready from a kernel of their own
 // (exponentials and logarithms of every token at once, not in this chain).  RPL >= ceil(d / 8); NJ =
@@ -262,7 +263,7 @@ extern "C" int fg_decay_chunk_states(float* chunks, const float* prod, float* st
 extern "C" int fg_decay_scan(const ScanArgs* args, int n_seqs, int act_dtype, hipStream_t stream) {
   if (n_seqs <= 0) return FG_OK;
   const ScanArgs& a = *args;
-  if (a.H <= 0 || a.d <= 0 || a.d > 256 || a.e <= 0 || a.H > 65535 || (a.e + 7) / 8 > 65535 || !a.qkv || !a.decay ||
+  if (a.H <= 0 || a.d <= 0 || a.d > 512 || a.e <= 0 || a.H > 65535 || (a.e + 7) / 8 > 65535 || !a.qkv || !a.decay ||
       !a.state || !a.slot_ids || !a.q_start || !a.out)
     return FG_ERR_ARG;
   dim3 grid(n_seqs, a.H, (a.e + 7) / 8);
@@ -274,7 +275,8 @@ extern "C" int fg_decay_scan(const ScanArgs* args, int n_seqs, int act_dtype, hi
     if (rpl <= 4) GO(TA, 4);     \
     else if (rpl <= 8) GO(TA, 8);   \
     else if (rpl <= 16) GO(TA, 16); \
-    else GO(TA, 32);             \
+    else if (rpl <= 32) GO(TA, 32); \
+    else GO(TA, 64);             \
   } while (0)
   if (act_dtype == FG_F32) LAUNCH(float);
   else if (act_dtype == FG_BF16) LAUNCH(bf16_t);

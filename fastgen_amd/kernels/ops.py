@@ -1298,7 +1298,7 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
     _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, H * e), "out must be contiguous float32 [T, H*e]")
     _i32(slot_ids, "slot_ids", n_seqs)
     _i32(q_start, "q_start", n_seqs + 1)
-    _need(d <= 256 and tau > 0, "at most 256 key channels a head; tau positive")
+    _need(d <= 512 and tau > 0, "at most 512 key channels a head; tau positive")
     a = _ScanArgs()
     a.qkv, a.row_stride, a.q_col, a.k_col, a.v_col = qkv.data_ptr(), qkv.stride(0), q_col, k_col, v_col
     # the decays of every token at once (exponentials and logarithms stay out of the chain of tokens)

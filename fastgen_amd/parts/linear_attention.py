@@ -33,9 +33,9 @@ class GatedLinearAttention(Mixer):
         self.tau = float(o["tau"])
         self.decay_rank = int(o["decay_rank"])
         self.eps = float(o["eps"])
-        if self.head_dim > 256 or self.v_head_dim > 1024:
+        if self.head_dim > 512 or self.v_head_dim > 1024:
             raise ValueError(f"{self.prefix}: heads of {self.head_dim} x {self.v_head_dim} are not supported"
-                             " (at most 256 key channels and 1024 value channels)")
+                             " (at most 512 key channels and 1024 value channels)")
         if not self.tau > 0:
             raise ValueError(f"{self.prefix}: tau must be positive")
         self.w_in: Optional[StreamedMatrix] = None
